@@ -1,0 +1,39 @@
+"""blockrank_amd: BlockRank block-sparse prefill attention and attention-score ranking on MI355X.
+
+Public surface (same names as the reference package exports for this path,
+src/blockrank/__init__.py:19-33):
+
+    register_blockrank_attention, register_triton_blockrank_attention   attention-interface hooks
+    compute_auxiliary_attention_loss                                    per-document scores
+
+plus the functional entry points ``blockrank_attention``, ``doc_scores``, ``last_block_logits`` and
+the ``BlockMask`` / ``LastBlockScores`` objects the hooks exchange.  Everything computes in
+hand-written HIP kernels (libblockrank_hip.so); there is no fallback implementation.
+"""
+from .attention import (
+    BlockMask,
+    LastBlockScores,
+    blockrank_attention,
+    blockrank_attention_forward,
+    blockrank_attention_mask,
+    doc_scores,
+    last_block_logits,
+    register_blockrank_attention,
+    register_triton_blockrank_attention,
+)
+from .losses import compute_auxiliary_attention_loss, rank_documents
+
+__all__ = [
+    "BlockMask",
+    "LastBlockScores",
+    "blockrank_attention",
+    "blockrank_attention_forward",
+    "blockrank_attention_mask",
+    "doc_scores",
+    "last_block_logits",
+    "register_blockrank_attention",
+    "register_triton_blockrank_attention",
+    "compute_auxiliary_attention_loss",
+    "rank_documents",
+]
+__version__ = "0.1.0"

@@ -1,0 +1,401 @@
+"""Hugging Face attention-interface hooks for BlockRank attention on MI355X.
+
+Mirrors the reference's plugin surface for this path:
+  * ``register_blockrank_attention()``          (src/blockrank/blockrank_std_attention.py:652-665)
+  * ``register_triton_blockrank_attention()``   (src/blockrank/blockrank_triton_kernel_attention.py:938-965)
+  * the attention hook ``fwd(module, query, key, value, attention_mask, scaling, dropout=0.0, **kwargs)
+    -> (attn_output (B, S, Nq, D), scores_or_None)`` (blockrank_std_attention.py:472-481, 648-650)
+  * the mask hook that turns the collate's (B, M, H) block mask into what the attention hook receives
+    as ``attention_mask`` (blockrank_std_attention.py:264-309).
+
+Every implementation name the reference registers is routed to the one HIP path; there is no eager,
+SDPA, flex or Triton code here and no fallback when the HIP library is absent.
+"""
+from __future__ import annotations
+
+import os
+import warnings
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+# Names the reference registers (blockrank_std_attention.py:654-665).
+STD_IMPL_NAMES = (
+    "default_blockrank",
+    "max-autotune_blockrank",
+    "eager_blockrank",
+    "flex_blockrank",
+    "sdpa_blockrank",
+    "sdpa_compiled_blockrank",
+)
+# blockrank_triton_kernel_attention.py:960-965
+TRITON_IMPL_NAMES = ("triton_blockrank", "triton_blockrank_compiled")
+
+_DTYPE_CODE = {torch.float32: _lib.BR_DTYPE_F32, torch.bfloat16: _lib.BR_DTYPE_BF16}
+
+
+def _env_flag(name: str) -> bool:
+    return os.environ.get(name, "0") not in ("", "0", "false", "False")
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class BlockMask:
+    """What the mask hook hands to the attention hook: the (B, M, H) real-token mask plus the device
+    plan built from it.
+
+    It stands where the reference passes a (B, 1, M, H, H) additive tensor
+    (blockrank_std_attention.py:293-309) and reports that shape, but holds B*M*H bytes instead of
+    B*M*H*H values; ``dense()`` materialises the reference tensor for callers that want it.  Plans
+    are built lazily per head layout and shared by every layer of a forward pass.
+    """
+
+    def __init__(self, valid: torch.Tensor, dtype: torch.dtype = torch.float32):
+        assert valid.dim() == 3, "block attention mask must be (B, M, H)"
+        if not valid.is_cuda:
+            raise RuntimeError("blockrank_amd runs on a GPU only: the block attention mask must be a CUDA/HIP tensor")
+        self.valid = valid.bool().contiguous()
+        self.dtype = dtype
+        self.B, self.M, self.H = valid.shape
+        self._plans: dict[tuple[int, int], torch.Tensor] = {}
+
+    # -- what the reference's 5-D tensor would answer ------------------------------------------
+    @property
+    def shape(self):
+        return torch.Size((self.B, 1, self.M, self.H, self.H))
+
+    @property
+    def device(self):
+        return self.valid.device
+
+    def dim(self) -> int:
+        return 5
+
+    def size(self, i: Optional[int] = None):
+        return self.shape if i is None else self.shape[i]
+
+    def to(self, *args, **kwargs):
+        return self
+
+    def dense(self, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """The reference's additive mask: 0 where key j of the block is real and j <= i, else
+        0.7 * finfo(dtype).min (blockrank_std_attention.py:297-307)."""
+        dtype = dtype or self.dtype
+        B, M, H = self.B, self.M, self.H
+        keep = self.valid.view(B, 1, M, 1, H) & torch.tril(torch.ones(H, H, dtype=torch.bool, device=self.valid.device))
+        neg = 0.7 * torch.finfo(dtype).min
+        return torch.where(keep, torch.zeros((), dtype=dtype, device=keep.device), torch.full((), neg, dtype=dtype, device=keep.device))
+
+    @classmethod
+    def from_dense(cls, mask5: torch.Tensor) -> "BlockMask":
+        """Recover the block mask from a reference-style (B, 1, M, H, H) additive tensor: the last
+        row of each H x H tile is zero exactly at the block's real keys."""
+        assert mask5.dim() == 5, "Attention mask must be 5D for BlockRank attention"
+        return cls(mask5[:, 0, :, -1, :] == 0, mask5.dtype)
+
+    # -- device plan --------------------------------------------------------------------------
+    def plan(self, Nq: int, Nkv: int) -> torch.Tensor:
+        key = (Nq, Nkv)
+        plan = self._plans.get(key)
+        if plan is None:
+            lib = _lib.load()
+            n = lib.br_plan_ints(self.B, self.M, self.H, Nq, Nkv)
+            assert n > 0, f"unsupported head layout: {Nq} query heads, {Nkv} kv heads"
+            with torch.cuda.device(self.valid.device):
+                plan = torch.empty(n, dtype=torch.int32, device=self.valid.device)
+                _lib.check(lib.br_plan_build(self.valid.data_ptr(), self.B, self.M, self.H, Nq, Nkv, plan.data_ptr(), n,
+                                             _stream_ptr(self.valid.device)))
+            if _env_flag("BLOCKRANK_AMD_DEBUG"):
+                # same role as the reference's _DEBUG left-padding check (blockrank_std_attention.py:146-148)
+                assert int(plan[4].item()) == 0, "Attention mask is not one contiguous span of real tokens per block"
+            self._plans[key] = plan
+        return plan
+
+    def block_lengths(self) -> torch.Tensor:
+        """(B, M) int32 number of real tokens per block."""
+        return self.valid.sum(-1, dtype=torch.int32)
+
+
+def blockrank_attention_mask(
+    batch_size=None,
+    cache_position=None,
+    kv_length=None,
+    kv_offset=0,
+    mask_function=None,
+    attention_mask: Optional[torch.Tensor] = None,
+    dtype: torch.dtype = torch.float32,
+    **kwargs,
+):
+    """Mask hook (AttentionMaskInterface).  Accepts both calling conventions of the transformers
+    library - the older positional ``cache_position`` one the reference is written against
+    (blockrank_std_attention.py:264-273) and the newer keyword one (``q_length``, ``q_offset``, ...),
+    and like the reference ignores everything except ``attention_mask`` (B, M, H) and ``dtype``.
+
+    Returns a BlockMask.  With BLOCKRANK_AMD_DENSE_MASK=1 it returns the reference's dense
+    (B, 1, M, H, H) tensor instead, which the attention hook also accepts."""
+    assert attention_mask is not None, "attention_mask must be provided for BlockRank attention"
+    assert attention_mask.dim() == 3, "BlockRank attention mask must be (B, M, H)"
+    bm = BlockMask(attention_mask, dtype)
+    if _env_flag("BLOCKRANK_AMD_DENSE_MASK"):
+        return bm.dense()
+    return bm
+
+
+def _as_block_mask(attention_mask) -> BlockMask:
+    assert attention_mask is not None, "BlockRank attention requires an attention mask"
+    if isinstance(attention_mask, BlockMask):
+        return attention_mask
+    assert len(attention_mask.shape) == 5, "Attention mask must be 5D for BlockRank attention"
+    cached = getattr(attention_mask, "_blockrank_block_mask", None)
+    if cached is None:
+        cached = BlockMask.from_dense(attention_mask)
+        try:
+            attention_mask._blockrank_block_mask = cached   # every layer of the forward reuses the plan
+        except Exception:
+            pass
+    return cached
+
+
+def _dense_last_dim(t: torch.Tensor, per16: int) -> torch.Tensor:
+    """The kernels read 16-byte pieces along the head dim: make it dense and the strides/pointer
+    16-byte multiples (a copy only if the caller's view is not already so)."""
+    if t.stride(-1) != 1 or any(s % per16 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+        t = t.contiguous()
+    return t
+
+
+def blockrank_attention(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    block_mask,
+    scaling: float,
+) -> torch.Tensor:
+    """Block-sparse prefill attention.  query (B, Nq, S, D), key/value (B, Nkv, S, D) with any
+    (batch, head, token) strides; block_mask a BlockMask, a (B, M, H) bool tensor, or the reference's
+    (B, 1, M, H, H) additive tensor.  Returns (B, S, Nq, D) contiguous, rows of padded slots zero.
+
+    Same result as sdpa_blockrank_attention_forward (blockrank_std_attention.py:503-650) on rows of
+    real tokens."""
+    if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
+        block_mask = BlockMask(block_mask, query.dtype)
+    bm = _as_block_mask(block_mask)
+    if not query.is_cuda:
+        raise RuntimeError("blockrank_amd runs on a GPU only (got CPU tensors); it has no CPU fallback")
+    B, Nq, S, D = query.shape
+    Nkv = key.shape[1]
+    M, H = bm.M, bm.H
+    assert H == S // M and M * H == S, f"Block size H={H} does not match MH // M = {S // M}"
+    assert key.shape == (B, Nkv, S, D) and value.shape == (B, Nkv, S, D), "key/value must be (B, Nkv, S, D)"
+    assert bm.B == B, "attention mask batch size does not match query"
+    if query.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
+    assert key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value must share a dtype"
+    if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
+        # same contract as the reference's kernelised path (blockrank_triton_kernel_attention.py:759-761)
+        raise NotImplementedError("Backward pass not implemented yet")
+    lib = _lib.load()
+    per16 = 16 // query.element_size()
+    q = _dense_last_dim(query, per16)
+    k = _dense_last_dim(key, per16)
+    v = _dense_last_dim(value, per16)
+    dev = query.device
+    with torch.cuda.device(dev):
+        plan = bm.plan(Nq, Nkv)
+        out = torch.empty((B, S, Nq, D), dtype=query.dtype, device=dev)
+        ws_bytes = lib.br_prefill_workspace_bytes(B, Nq, Nkv, D)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        out_strides = _lib._I64x3(S * Nq * D, D, Nq * D)
+        _lib.check(lib.br_prefill_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
+            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), out_strides, float(scaling), _DTYPE_CODE[query.dtype],
+            ws.data_ptr(), ws_bytes, _stream_ptr(dev)))
+    return out
+
+
+class LastBlockScores:
+    """Handle returned in place of the reference's s_last tensor (B, Nq, R, S)
+    (blockrank_std_attention.py:639-645): it keeps the layer's query/key tensors and the block mask so
+    that per-document scores are computed by the fused kernel without writing the logits out.
+
+    ``compute_auxiliary_attention_loss`` of this package accepts it directly; ``dense()`` produces the
+    reference tensor for anything else."""
+
+    def __init__(self, query, key, block_mask: BlockMask, scaling: float, num_rows: int, scaled: bool = True):
+        self.query, self.key, self.block_mask = query, key, block_mask
+        self.scaling, self.R, self.scaled = float(scaling), int(num_rows), scaled
+        B, Nq, S, D = query.shape
+        self.shape = torch.Size((B, Nq, self.R, S))
+        self.device, self.dtype = query.device, query.dtype
+
+    def dim(self) -> int:
+        return 4
+
+    def size(self, i=None):
+        return self.shape if i is None else self.shape[i]
+
+    def _rows_default(self) -> torch.Tensor:
+        H = self.block_mask.H
+        return (torch.arange(H - self.R, H, dtype=torch.int32, device=self.device)[None]).expand(self.shape[0], self.R).contiguous()
+
+    def dense(self, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """(B, Nq, R, S) logits + additive mask, fp32 unless ``dtype`` is given."""
+        out = last_block_logits(self.query, self.key, self.block_mask, self._rows_default(),
+                                self.scaling if self.scaled else 1.0, neg=0.7 * torch.finfo(self.dtype).min)
+        return out if dtype is None else out.to(dtype)
+
+    def doc_scores(self, rows: torch.Tensor, temperature: float = 0.05, head_reduce: str = "mean", row_reduce: str = "mean",
+                   return_probs: bool = False):
+        """Per-document scores for ``rows`` (B, R') positions inside the query block (0..H-1)."""
+        return doc_scores(self.query, self.key, self.block_mask, rows, self.scaling if self.scaled else 1.0,
+                          temperature=temperature, head_reduce=head_reduce, row_reduce=row_reduce, return_probs=return_probs)
+
+
+def _score_args(query, key, block_mask, rows):
+    if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
+        block_mask = BlockMask(block_mask, query.dtype)
+    bm = _as_block_mask(block_mask)
+    if not query.is_cuda:
+        raise RuntimeError("blockrank_amd runs on a GPU only (got CPU tensors); it has no CPU fallback")
+    B, Nq, S, D = query.shape
+    Nkv = key.shape[1]
+    assert bm.M * bm.H == S, "attention mask does not match the sequence length"
+    if query.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
+    assert rows.dim() == 2 and rows.shape[0] == B, "rows must be (B, R)"
+    per16 = 16 // query.element_size()
+    q = _dense_last_dim(query, per16)
+    k = _dense_last_dim(key, per16)
+    rows = rows.to(device=query.device, dtype=torch.int32).contiguous()
+    return bm, q, k, rows, (B, Nq, Nkv, S, D)
+
+
+def doc_scores(query, key, block_mask, rows, scaling: float, temperature: float = 0.05, head_reduce: str = "mean",
+               row_reduce: str = "mean", return_probs: bool = False):
+    """Fused per-document relevance: for every (head, chosen query-block row) a softmax of
+    scaling*q.k over all real document tokens, summed per document, reduced over heads and rows and
+    divided by the temperature.  Equals compute_auxiliary_attention_loss(s_last, ..., answer_ids=None,
+    return_logits=True) (src/blockrank/losses.py:37-78) with rows = the bracket row and the one before.
+
+    rows: (B, R) positions inside the query block (0..H-1), R <= 16.  Returns (B, M-2) fp32, and the
+    (B, Nq, R, M-2) per-head probabilities too if return_probs."""
+    bm, q, k, rows, (B, Nq, Nkv, S, D) = _score_args(query, key, block_mask, rows)
+    R = rows.shape[1]
+    assert bm.M >= 3, "per-document scores need at least one document block"
+    assert head_reduce in ("mean", "sum") and row_reduce in ("mean", "sum")
+    out_scale = 1.0 / temperature
+    if head_reduce == "mean":
+        out_scale /= Nq
+    if row_reduce == "mean":
+        out_scale /= R
+    lib = _lib.load()
+    dev = query.device
+    with torch.cuda.device(dev):
+        plan = bm.plan(Nq, Nkv)
+        scores = torch.empty((B, bm.M - 2), dtype=torch.float32, device=dev)
+        probs = torch.empty((B, Nq, R, bm.M - 2), dtype=torch.float32, device=dev) if return_probs else None
+        ws_bytes = lib.br_doc_scores_workspace_bytes(B, Nq, bm.M, R)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        _lib.check(lib.br_doc_scores(
+            q.data_ptr(), k.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, B, Nq, Nkv, bm.M, bm.H, D,
+            _lib.strides3(q), _lib.strides3(k), float(scaling), float(out_scale), _DTYPE_CODE[query.dtype],
+            scores.data_ptr(), probs.data_ptr() if probs is not None else None, ws.data_ptr(), ws_bytes, _stream_ptr(dev)))
+    return (scores, probs) if return_probs else scores
+
+
+def last_block_logits(query, key, block_mask, rows, scaling: float, neg: Optional[float] = None) -> torch.Tensor:
+    """The reference's s_last: (B, Nq, R, S) fp32 = scaling*q.k + (0 | neg) for the given query-block
+    rows against every key slot (blockrank_std_attention.py:233, 259, 639-645)."""
+    bm, q, k, rows, (B, Nq, Nkv, S, D) = _score_args(query, key, block_mask, rows)
+    R = rows.shape[1]
+    if neg is None:
+        neg = 0.7 * torch.finfo(query.dtype).min
+    lib = _lib.load()
+    dev = query.device
+    with torch.cuda.device(dev):
+        plan = bm.plan(Nq, Nkv)
+        out = torch.empty((B, Nq, R, S), dtype=torch.float32, device=dev)
+        _lib.check(lib.br_last_block_logits(
+            q.data_ptr(), k.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, B, Nq, Nkv, bm.M, bm.H, D,
+            _lib.strides3(q), _lib.strides3(k), float(scaling), float(neg), _DTYPE_CODE[query.dtype], out.data_ptr(),
+            _stream_ptr(dev)))
+    return out
+
+
+def blockrank_attention_forward(
+    module,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attention_mask,
+    scaling: float,
+    dropout: float = 0.0,
+    **kwargs,
+):
+    """Attention hook (AttentionInterface).  Same contract as the reference's forwards
+    (blockrank_std_attention.py:472-650, blockrank_triton_kernel_attention.py:798-884):
+
+      query (B, Nq, S, D), key/value (B, Nkv, S, D), attention_mask from the mask hook (a BlockMask, or
+      the reference's (B, 1, M, H, H) tensor); returns (attn_output (B, S, Nq, D), scores or None).
+
+    Scores are returned when ``layers_to_return_scores`` contains ``module.layer_idx`` or, without
+    that list, when ``return_last_block_attn_scores`` is true (:625-635), for the last
+    ``num_last_queries`` (default 16) rows of the query block (:637-645).  They come back as a
+    LastBlockScores handle (scaled logits, the eager/Triton convention); pass
+    ``materialize_scores=True`` or set BLOCKRANK_AMD_DENSE_SCORES=1 for the fp32 tensor itself, and
+    ``unscaled_scores=True`` for the literal SDPA function's unscaled variant (:537, :643).
+    """
+    assert attention_mask is not None, "BlockRank attention requires an attention mask"
+    bm = _as_block_mask(attention_mask)
+    B, Nq, S, D = query.shape
+    assert bm.H == S // bm.M, f"Block size H={bm.H} does not match MH // M = {S // bm.M}"
+    groups = getattr(module, "num_key_value_groups", None)
+    if groups is not None:
+        assert key.shape[1] * groups == Nq, "num_key_value_groups does not match the query/key head counts"
+    if dropout > 0.0 and getattr(module, "training", False):
+        warnings.warn("Dropout is not supported in kernelized BlockRank attention, ignoring dropout parameter")
+
+    out = blockrank_attention(query, key, value, bm, scaling)
+    if bm.M == 1:
+        return out, None
+
+    layers = kwargs.get("layers_to_return_scores", None)
+    if layers is not None:
+        layer_idx = getattr(module, "layer_idx", None)
+        want = layer_idx is not None and layer_idx in layers
+    else:
+        want = kwargs.get("return_last_block_attn_scores", False)
+    if not want:
+        return out, None
+    num_last = kwargs.get("num_last_queries", 16)
+    R = num_last if bm.H >= num_last else bm.H
+    handle = LastBlockScores(query, key, bm, scaling, R, scaled=not kwargs.get("unscaled_scores", False))
+    if kwargs.get("materialize_scores", False) or _env_flag("BLOCKRANK_AMD_DENSE_SCORES"):
+        return out, handle.dense()
+    return out, handle
+
+
+def _register(names) -> None:
+    try:
+        from transformers import AttentionInterface, AttentionMaskInterface
+    except ImportError as e:  # same failure mode as blockrank_triton_kernel_attention.py:951-955
+        raise ImportError("Transformers is not available. Please install it with: pip install transformers") from e
+    for name in names:
+        AttentionInterface.register(name, blockrank_attention_forward)
+        AttentionMaskInterface.register(name, blockrank_attention_mask)
+
+
+def register_blockrank_attention() -> None:
+    """Register the implementation names of blockrank_std_attention.py:652-665, all served by the
+    HIP path."""
+    _register(STD_IMPL_NAMES)
+
+
+def register_triton_blockrank_attention() -> None:
+    """Register the implementation names of blockrank_triton_kernel_attention.py:938-965, served by
+    the HIP path (nothing here uses Triton)."""
+    _register(TRITON_IMPL_NAMES)

@@ -1,0 +1,242 @@
+// extern "C" entry points of libblockrank_hip.so: argument checks, geometry selection, launches.
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../../include/blockrank_hip.h"
+#include "br_common.h"
+
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int B, int M, int H, int T, int* plan,
+                    hipStream_t stream);
+int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream);
+int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream);
+int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
+                         float* probs, const long long* sq, const long long* sk, int B, int Nq, int Nkv, int M, int H, int D,
+                         int R, int T, float scale, float out_scale, int dtype, hipStream_t stream);
+int br_launch_last_logits(const void* q, const void* k, const int* plan, const int* rows, float* logits, const long long* sq,
+                          const long long* sk, int B, int Nq, int Nkv, int M, int H, int D, int R, int T, float scale,
+                          float neg, int dtype, hipStream_t stream);
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// Head layout -> workgroup shape.  A workgroup carries NW row blocks of 32 query rows: Gw heads of
+// one kv head's group times tpb 32-token sub-blocks.
+bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW) {
+    if (Nq <= 0 || Nkv <= 0 || Nq % Nkv) return false;
+    const int G = Nq / Nkv;
+    int Gw = 1;
+    for (int d = 1; d <= 8 && d <= G; ++d)
+        if (G % d == 0) Gw = d;
+    int nw, tpb;
+    switch (Gw) {
+        case 1: nw = 4; tpb = 4; break;
+        case 2: nw = 4; tpb = 2; break;
+        case 3: nw = 6; tpb = 2; break;
+        case 4: nw = 4; tpb = 1; break;
+        default: nw = Gw; tpb = 1; break;
+    }
+    // experiment knob: BLOCKRANK_WIDE_TILES=1 doubles the tokens per tile where 8 waves allow it
+    static const bool wide = getenv("BLOCKRANK_WIDE_TILES") && atoi(getenv("BLOCKRANK_WIDE_TILES")) != 0;
+    if (wide && nw == 4) {
+        nw = 8;
+        tpb *= 2;
+    }
+    g->G = G;
+    g->Gw = Gw;
+    g->tpb = tpb;
+    g->HGS = G / Gw;
+    g->NHG = Nkv * g->HGS;
+    *NW = nw;
+    return true;
+}
+
+int n_compute_units() {
+    static thread_local int cached_dev = -1, cached_cu = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (dev != cached_dev) {
+        int cu = 0;
+        if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached_dev = dev;
+        cached_cu = cu;
+    }
+    return cached_cu;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(BR_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+    return BR_OK;
+}
+
+int check_common(int B, int Nq, int Nkv, int M, int H, int D, int dtype) {
+    if (B <= 0 || M <= 0 || H <= 0) return fail(BR_ERR_ARG, "B, M and H must be positive (got %d, %d, %d)", B, M, H);
+    if (Nq <= 0 || Nkv <= 0 || Nq % Nkv) return fail(BR_ERR_ARG, "Nq=%d must be a positive multiple of Nkv=%d", Nq, Nkv);
+    if (D != 64 && D != 128) return fail(BR_ERR_ARG, "head dim %d not supported (64 or 128)", D);
+    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "dtype %d not supported", dtype);
+    return BR_OK;
+}
+
+int check_strides(const char* name, const int64_t* s, int dtype) {
+    if (!s) return fail(BR_ERR_ARG, "%s strides are null", name);
+    const int per16 = dtype == BR_DTYPE_F32 ? 4 : 8;
+    for (int i = 0; i < 3; ++i)
+        if (s[i] < 0 || s[i] % per16) return fail(BR_ERR_ARG, "%s stride %d = %lld is not a multiple of 16 bytes", name, i, (long long)s[i]);
+    return BR_OK;
+}
+
+size_t slots_total(int B, const BrGeom& g) { return (size_t)B * BR_SLOTS_PER_SEQ * g.NHG; }
+
+}  // namespace
+
+extern "C" {
+
+int br_version(void) { return 100; }
+
+const char* br_last_error(void) { return g_err; }
+
+int br_tile_tokens(int Nq, int Nkv) {
+    BrGeom g;
+    int nw;
+    if (!make_geom(Nq, Nkv, &g, &nw)) return 0;
+    return br_tokens_per_tile(g);
+}
+
+size_t br_plan_ints(int B, int M, int H, int Nq, int Nkv) {
+    int T = br_tile_tokens(Nq, Nkv);
+    if (T == 0 || B <= 0 || M <= 0 || H <= 0) return 0;
+    return br_plan_total_ints(B, M, H, T);
+}
+
+static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded, int B, int M, int H, int Nq, int Nkv,
+                      int32_t* plan, size_t plan_ints, void* stream) {
+    if (B <= 0 || M <= 0 || H <= 0) return fail(BR_ERR_ARG, "B, M and H must be positive (got %d, %d, %d)", B, M, H);
+    int T = br_tile_tokens(Nq, Nkv);
+    if (T == 0) return fail(BR_ERR_ARG, "Nq=%d must be a positive multiple of Nkv=%d", Nq, Nkv);
+    if (!plan || (!valid && !lens)) return fail(BR_ERR_ARG, "null pointer");
+    if (!aligned16(plan)) return fail(BR_ERR_ARG, "plan buffer must be 16-byte aligned");
+    if (plan_ints < br_plan_total_ints(B, M, H, T))
+        return fail(BR_ERR_SPACE, "plan buffer holds %zu ints, %zu needed", plan_ints, br_plan_total_ints(B, M, H, T));
+    br_launch_plan(valid, lens, left_padded, B, M, H, T, plan, static_cast<hipStream_t>(stream));
+    return check_launch("plan launch");
+}
+
+int br_plan_build(const uint8_t* valid, int B, int M, int H, int Nq, int Nkv, int32_t* plan, size_t plan_ints, void* stream) {
+    if (!valid) return fail(BR_ERR_ARG, "attention mask must be provided");
+    return plan_build(valid, nullptr, 1, B, M, H, Nq, Nkv, plan, plan_ints, stream);
+}
+
+int br_plan_build_from_lengths(const int32_t* lens, int left_padded, int B, int M, int H, int Nq, int Nkv, int32_t* plan,
+                               size_t plan_ints, void* stream) {
+    if (!lens) return fail(BR_ERR_ARG, "block lengths must be provided");
+    return plan_build(nullptr, lens, left_padded, B, M, H, Nq, Nkv, plan, plan_ints, stream);
+}
+
+size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
+    BrGeom g;
+    int nw;
+    if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || D <= 0) return 0;
+    size_t rows = slots_total(B, g) * (size_t)nw * BR_RB;
+    return rows * (size_t)(D + 2) * sizeof(float);
+}
+
+int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
+                   int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                   const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
+    if (rc) return rc;
+    if (!q || !k || !v || !out || !plan) return fail(BR_ERR_ARG, "null pointer");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(plan) || !aligned16(workspace))
+        return fail(BR_ERR_ARG, "q, k, v, out, plan and workspace must be 16-byte aligned");
+    if ((rc = check_strides("q", q_strides, dtype)) || (rc = check_strides("k", k_strides, dtype)) ||
+        (rc = check_strides("v", v_strides, dtype)) || (rc = check_strides("out", out_strides, dtype)))
+        return rc;
+    BrGeom g;
+    int nw;
+    make_geom(Nq, Nkv, &g, &nw);
+    const size_t need = br_prefill_workspace_bytes(B, Nq, Nkv, D);
+    if (!workspace || workspace_bytes < need) return fail(BR_ERR_SPACE, "workspace holds %zu bytes, %zu needed", workspace_bytes, need);
+    const int n_cu = n_compute_units();
+    if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
+
+    BrPrefillParams p;
+    p.q = q; p.k = k; p.v = v; p.out = out; p.plan = plan;
+    const size_t rows = slots_total(B, g) * (size_t)nw * BR_RB;
+    p.part_o = static_cast<float*>(workspace);
+    p.part_ml = p.part_o + rows * D;
+    p.sq_b = q_strides[0]; p.sq_h = q_strides[1]; p.sq_t = q_strides[2];
+    p.sk_b = k_strides[0]; p.sk_h = k_strides[1]; p.sk_t = k_strides[2];
+    p.sv_b = v_strides[0]; p.sv_h = v_strides[1]; p.sv_t = v_strides[2];
+    p.so_b = out_strides[0]; p.so_h = out_strides[1]; p.so_t = out_strides[2];
+    p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H;
+    p.geom = g;
+    p.scale_log2 = scale * 1.4426950408889634f;
+    int combine_grid = br_plan_max_comb(B) * g.NHG;
+    if (combine_grid < B * M) combine_grid = B * M;
+    if (combine_grid > 4 * n_cu) combine_grid = 4 * n_cu;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s)
+                                     : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s);
+    if (lrc) return fail(BR_ERR_ARG, "no kernel for head dim %d with %d query heads per kv head", D, g.G);
+    return check_launch("prefill launch");
+}
+
+size_t br_doc_scores_workspace_bytes(int B, int Nq, int M, int R) {
+    if (B <= 0 || Nq <= 0 || M < 3 || R <= 0) return 0;
+    return (size_t)B * Nq * R * (M - 2) * 2 * sizeof(float);
+}
+
+static int check_scores(const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B, int Nq, int Nkv,
+                        int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, int dtype) {
+    int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
+    if (rc) return rc;
+    if (R <= 0 || R > 16) return fail(BR_ERR_ARG, "R=%d rows not supported (1..16)", R);
+    if (!q || !k || !plan || !rows) return fail(BR_ERR_ARG, "null pointer");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(plan)) return fail(BR_ERR_ARG, "q, k and plan must be 16-byte aligned");
+    if ((rc = check_strides("q", q_strides, dtype)) || (rc = check_strides("k", k_strides, dtype))) return rc;
+    return BR_OK;
+}
+
+int br_doc_scores(const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B, int Nq, int Nkv, int M,
+                  int H, int D, const int64_t* q_strides, const int64_t* k_strides, float scale, float out_scale, int dtype,
+                  float* scores, float* probs, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_scores(q, k, plan, rows, R, B, Nq, Nkv, M, H, D, q_strides, k_strides, dtype);
+    if (rc) return rc;
+    if (M < 3) return fail(BR_ERR_ARG, "per-document scores need at least one document block (M=%d)", M);
+    if (!scores) return fail(BR_ERR_ARG, "null pointer");
+    const size_t need = br_doc_scores_workspace_bytes(B, Nq, M, R);
+    if (!workspace || workspace_bytes < need) return fail(BR_ERR_SPACE, "workspace holds %zu bytes, %zu needed", workspace_bytes, need);
+    const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]};
+    const long long sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
+    br_launch_doc_scores(q, k, plan, rows, static_cast<float*>(workspace), scores, probs, sq, sk, B, Nq, Nkv, M, H, D, R,
+                         br_tile_tokens(Nq, Nkv), scale, out_scale, dtype, static_cast<hipStream_t>(stream));
+    return check_launch("score launch");
+}
+
+int br_last_block_logits(const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B, int Nq, int Nkv,
+                         int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, float scale, float neg,
+                         int dtype, float* logits, void* stream) {
+    int rc = check_scores(q, k, plan, rows, R, B, Nq, Nkv, M, H, D, q_strides, k_strides, dtype);
+    if (rc) return rc;
+    if (!logits) return fail(BR_ERR_ARG, "null pointer");
+    const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]};
+    const long long sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
+    br_launch_last_logits(q, k, plan, rows, logits, sq, sk, B, Nq, Nkv, M, H, D, R, br_tile_tokens(Nq, Nkv), scale, neg, dtype,
+                          static_cast<hipStream_t>(stream));
+    return check_launch("logits launch");
+}
+
+}  // extern "C"

@@ -1,0 +1,159 @@
+// Shared definitions for the BlockRank gfx950 kernels: the block table, the request plan (work
+// items for the persistent prefill kernel), the key/value tile walk and the row mapping that the
+// bf16 MFMA kernel, the fp32 kernel and the combine kernel all use.
+//
+// Vocabulary (the reference's): a sequence is M blocks of padded length H; block 0 is the
+// instruction prefix, blocks 1..M-2 are documents, block M-1 is the query.  Each block holds one
+// contiguous span of real tokens [start, start+len) inside its H slots (left padding puts it at the
+// end).  Every position used by the kernels is "valid-relative": 0 is the block's first real token.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define BR_BN 64              // keys per key/value tile
+#define BR_RB 32              // query rows per wave (one 32x32 MFMA row block)
+#define BR_SLOTS_PER_SEQ 32   // split-KV partial slots available to one sequence's query block
+#define BR_MIN_CHUNK 4        // a split of the query block's key walk covers at least this many tiles
+
+// Plan buffer (int32): [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][items 8*max_items][comb 4*max_comb]
+#define BR_PLAN_HDR 16
+enum BrPlanHeader {
+    BR_PH_NITEMS = 0,     // number of work items (per head group)
+    BR_PH_NCOMB = 1,      // number of combine entries (per head group)
+    BR_PH_TICKET = 2,     // persistent-kernel ticket counter (zero between launches)
+    BR_PH_DONE = 3,       // workgroups that have left the persistent loop (zero between launches)
+    BR_PH_NONCONTIG = 4,  // set to 1 if some block's real tokens are not one contiguous span
+    BR_PH_MAX_ITEMS = 5,
+    BR_PH_MAX_COMB = 6,
+    BR_PH_T = 7,          // tokens per query tile the plan was built for
+};
+
+// One unit of prefill work: query tile [t0, t0+T) of block m of sequence b, restricted to a range
+// of its key/value tile walk.  li0/kt0 locate the first tile (walk-list position, tile inside it),
+// ntiles is how many tiles to process (INT_MAX = to the end).  slot < 0: the item owns its rows and
+// writes the final output; slot >= 0: it writes an unnormalised partial into that slot.
+struct BrItem {
+    int b, m, t0, li0, kt0, ntiles, slot, pad;
+};
+struct BrComb {
+    int b, t0, slot0, nsplit;
+};
+
+struct BrPlanView {
+    const int* hdr;
+    const int* start;   // B*M
+    const int* len;     // B*M
+    const BrItem* items;
+    const BrComb* comb;
+};
+
+__host__ __device__ inline size_t br_plan_off_start() { return BR_PLAN_HDR; }
+__host__ __device__ inline size_t br_plan_off_len(int B, int M) { return BR_PLAN_HDR + (size_t)B * M; }
+__host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M; }
+__host__ __device__ inline size_t br_plan_off_items(int B, int M) {
+    size_t o = BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B;
+    return (o + 7) & ~(size_t)7;   // 32-byte aligned so an item is two 16-byte loads
+}
+__host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
+    int qt = (H + T - 1) / T;
+    int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
+    return B * ((M > 1 ? (M - 1) * qt : 0) + last);
+}
+__host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }
+__host__ __device__ inline size_t br_plan_off_comb(int B, int M, int H, int T) {
+    return br_plan_off_items(B, M) + 8 * (size_t)br_plan_max_items(B, M, H, T);
+}
+__host__ __device__ inline size_t br_plan_total_ints(int B, int M, int H, int T) {
+    return br_plan_off_comb(B, M, H, T) + 4 * (size_t)br_plan_max_comb(B);
+}
+
+__device__ inline BrPlanView br_plan_view(const int* plan, int B, int M, int H, int T) {
+    BrPlanView v;
+    v.hdr = plan;
+    v.start = plan + br_plan_off_start();
+    v.len = plan + br_plan_off_len(B, M);
+    v.items = reinterpret_cast<const BrItem*>(plan + br_plan_off_items(B, M));
+    v.comb = reinterpret_cast<const BrComb*>(plan + br_plan_off_comb(B, M, H, T));
+    return v;
+}
+
+// Number of earlier blocks a query block m attends to in full: none for the prefix, the prefix for
+// a document, every earlier block for the query block (which is also block 0 when M == 1).
+__host__ __device__ inline int br_prev_blocks(int m, int M) {
+    if (m == 0) return 0;
+    return m == M - 1 ? M - 1 : 1;
+}
+
+// Walk over the key/value tiles one query tile sees: all tiles of blocks 0..pe-1 (full visibility),
+// then the tiles of its own block up to the diagonal.  Every field is uniform across the workgroup.
+struct BrTile {
+    int blk;      // block the tile's keys live in
+    int kt;       // tile index inside that block (valid-relative key kt*BR_BN is its first key)
+    int nvalid;   // real keys in the tile (1..BR_BN)
+    int self;     // 1 if the keys belong to the query tile's own block (causal rule applies)
+};
+
+struct BrWalk {
+    const int* len;   // lengths of this sequence's blocks
+    int pe, m, self_end;
+    int li, kt, left;
+
+    __device__ void init(const int* len_b, int m_, int M, int self_end_, int li0, int kt0, int ntiles) {
+        len = len_b;
+        m = m_;
+        pe = br_prev_blocks(m_, M);
+        self_end = self_end_;
+        li = li0;
+        kt = kt0;
+        left = ntiles;
+    }
+    __device__ bool next(BrTile& t) {
+        if (left <= 0) return false;
+        while (li <= pe) {
+            int L = li < pe ? len[li] : self_end;
+            int k0 = kt * BR_BN;
+            if (k0 < L) {
+                t.blk = li < pe ? li : m;
+                t.kt = kt;
+                t.nvalid = L - k0 < BR_BN ? L - k0 : BR_BN;
+                t.self = li == pe;
+                ++kt;
+                --left;
+                return true;
+            }
+            ++li;
+            kt = 0;
+        }
+        return false;
+    }
+};
+
+// Row mapping shared by every kernel that touches a work item: a workgroup of NW "row blocks" of 32
+// query rows covers Gw = NW / tpb heads x T = 32 * tpb tokens.  Row block r is head r / tpb of the
+// group and token sub-block r % tpb.  hg enumerates (kv head, head sub-group).
+struct BrGeom {
+    int G;      // query heads per kv head
+    int Gw;     // heads one workgroup covers
+    int tpb;    // 32-token sub-blocks per query tile
+    int HGS;    // head sub-groups per kv head = G / Gw
+    int NHG;    // head groups in total = Nkv * HGS
+};
+
+__host__ __device__ inline int br_tokens_per_tile(const BrGeom& g) { return g.tpb * BR_RB; }
+
+struct BrPrefillParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* out;
+    const int* plan;
+    float* part_o;    // split-KV partial outputs: [slot][NW*32 rows][D] fp32, unnormalised
+    float* part_ml;   // [slot][NW*32 rows][2]: running max (log2 domain) and denominator
+    long long sq_b, sq_h, sq_t;   // element strides of q for (batch, head, token); the last dim is dense
+    long long sk_b, sk_h, sk_t;
+    long long sv_b, sv_h, sv_t;
+    long long so_b, so_h, so_t;
+    int B, Nq, Nkv, M, H;
+    BrGeom geom;
+    float scale_log2;  // softmax scale * log2(e)
+};

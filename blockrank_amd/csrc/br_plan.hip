@@ -1,0 +1,221 @@
+// Request plan: turns the (B, M, H) block mask into the block table (start, len per block) and the
+// work-item list the persistent prefill kernel consumes.  Built on the device with no host
+// synchronisation, once per forward pass (the block structure is the same for every layer).
+//
+// The additive 5-D mask of the reference (blockrank_std_attention.py:293-309) carries exactly this
+// information: which keys of each block are real.  Everything else (causality inside a block, which
+// earlier blocks a block may see) follows from the block index, so the kernels never read a mask.
+#include "br_common.h"
+
+namespace {
+
+constexpr int kPlanThreads = 1024;
+
+// One wave per block: count real tokens, find the first and the last.  len is written negated
+// (-1 - count) when the real tokens are not one contiguous span; the plan kernel repairs the sign
+// and raises the header flag.
+__global__ __launch_bounds__(256) void br_block_table_kernel(const uint8_t* __restrict__ valid, int BM, int H,
+                                                             int* __restrict__ start, int* __restrict__ len) {
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    if (wave >= BM) return;
+    const uint8_t* row = valid + (size_t)wave * H;
+    int cnt = 0, first = H, last = -1;
+    for (int j = lane; j < H; j += 64) {
+        if (row[j]) {
+            ++cnt;
+            first = j < first ? j : first;
+            last = j > last ? j : last;
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        cnt += __shfl_xor(cnt, o);
+        int f = __shfl_xor(first, o);
+        int l = __shfl_xor(last, o);
+        first = f < first ? f : first;
+        last = l > last ? l : last;
+    }
+    if (lane == 0) {
+        bool contiguous = cnt == 0 || (last - first + 1 == cnt);
+        start[wave] = cnt == 0 ? 0 : first;
+        len[wave] = contiguous ? cnt : -1 - cnt;
+    }
+}
+
+__device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Exclusive scan of one int per thread over the workgroup (kPlanThreads entries); returns the
+// exclusive prefix and leaves the total in *total.
+__device__ int block_exclusive_scan(int x, int* sh, int* total) {
+    const int tid = threadIdx.x;
+    sh[tid] = x;
+    __syncthreads();
+    for (int o = 1; o < kPlanThreads; o <<= 1) {
+        int y = tid >= o ? sh[tid - o] : 0;
+        __syncthreads();
+        sh[tid] += y;
+        __syncthreads();
+    }
+    int incl = sh[tid];
+    *total = sh[kPlanThreads - 1];
+    __syncthreads();
+    return incl - x;
+}
+
+// Split count for query tile tt of the query block: enough splits that each covers about
+// BR_MIN_CHUNK key tiles, limited so that all tiles of the block fit the sequence's slot budget.
+__device__ inline int splits_for(int ntiles, int ns_cap) {
+    int ns = ceil_div(ntiles, BR_MIN_CHUNK);
+    ns = ns < 1 ? 1 : ns;
+    return ns > ns_cap ? ns_cap : ns;
+}
+
+__global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T) {
+    __shared__ int sh[kPlanThreads];
+    __shared__ int s_bad;
+    const int tid = threadIdx.x;
+    int* hdr = plan;
+    int* start = plan + br_plan_off_start();
+    int* len = plan + br_plan_off_len(B, M);
+    int* prev_tiles = plan + br_plan_off_prev(B, M);
+    BrItem* items = reinterpret_cast<BrItem*>(plan + br_plan_off_items(B, M));
+    BrComb* comb = reinterpret_cast<BrComb*>(plan + br_plan_off_comb(B, M, H, T));
+    (void)start;
+
+    if (tid < BR_PLAN_HDR) hdr[tid] = 0;
+    if (tid == 0) s_bad = 0;
+    __syncthreads();
+    const int BM = B * M;
+    for (int p = tid; p < BM; p += kPlanThreads) {
+        int l = len[p];
+        if (l < 0) {
+            len[p] = -1 - l;
+            s_bad = 1;
+        }
+    }
+    __syncthreads();
+    for (int b = tid; b < B; b += kPlanThreads) {
+        int s = 0;
+        for (int m = 0; m < M - 1; ++m) s += ceil_div(len[b * M + m], BR_BN);
+        prev_tiles[b] = s;
+    }
+    __syncthreads();
+
+    // Pairs are visited sequence by sequence, the query block first: its split items are the long
+    // ones and go to the front of each sequence's run of items.
+    int base_items = 0, base_comb = 0;
+    for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
+        const int p = p0 + tid;
+        int n_items = 0, n_comb = 0;
+        int b = 0, m = 0, L = 0, nq = 0, ns_cap = 1, pt = 0;
+        bool is_last = false;
+        if (p < BM) {
+            b = p / M;
+            int jj = p - b * M;
+            m = jj == 0 ? M - 1 : jj - 1;
+            is_last = jj == 0;
+            L = len[b * M + m];
+            nq = ceil_div(L, T);
+            if (is_last) {
+                pt = M > 1 ? prev_tiles[b] : 0;
+                ns_cap = nq > 0 ? BR_SLOTS_PER_SEQ / nq : 1;
+                ns_cap = ns_cap < 1 ? 1 : ns_cap;
+                for (int tt = 0; tt < nq; ++tt) {
+                    int e = (tt + 1) * T < L ? (tt + 1) * T : L;
+                    int ns = splits_for(pt + ceil_div(e, BR_BN), ns_cap);
+                    n_items += ns;
+                    n_comb += ns > 1;
+                }
+            } else {
+                n_items = nq;
+            }
+        }
+        int tot_i, tot_c;
+        int off_i = base_items + block_exclusive_scan(n_items, sh, &tot_i);
+        int off_c = base_comb + block_exclusive_scan(n_comb, sh, &tot_c);
+        base_items += tot_i;
+        base_comb += tot_c;
+        if (p < BM) {
+            if (!is_last) {
+                const int pe = br_prev_blocks(m, M);
+                for (int tt = 0; tt < nq; ++tt) {
+                    BrItem it;
+                    it.b = b; it.m = m; it.t0 = tt * T; it.li0 = 0; it.kt0 = 0;
+                    it.ntiles = 0x7fffffff; it.slot = -1; it.pad = pe;
+                    items[off_i + tt] = it;
+                }
+            } else {
+                const int pe = br_prev_blocks(m, M);
+                const int* len_b = len + b * M;
+                int slot = 0;
+                for (int tt = 0; tt < nq; ++tt) {
+                    int e = (tt + 1) * T < L ? (tt + 1) * T : L;
+                    int nself = ceil_div(e, BR_BN);
+                    int nt = pt + nself;
+                    int ns = splits_for(nt, ns_cap);
+                    if (ns > 1) {
+                        BrComb c;
+                        c.b = b; c.t0 = tt * T; c.slot0 = slot; c.nsplit = ns;
+                        comb[off_c++] = c;
+                    }
+                    // walk-list cursor: position li, tiles before it cum
+                    int li = 0, cum = 0;
+                    for (int s = 0; s < ns; ++s) {
+                        int lo = (int)((long long)s * nt / ns);
+                        int hi = (int)((long long)(s + 1) * nt / ns);
+                        for (;;) {
+                            int tl = li < pe ? ceil_div(len_b[li], BR_BN) : nself;
+                            if (li >= pe || lo < cum + tl) break;
+                            cum += tl;
+                            ++li;
+                        }
+                        BrItem it;
+                        it.b = b; it.m = m; it.t0 = tt * T; it.li0 = li; it.kt0 = lo - cum;
+                        it.ntiles = hi - lo; it.slot = ns > 1 ? slot + s : -1; it.pad = pe;
+                        items[off_i++] = it;
+                    }
+                    if (ns > 1) slot += ns;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        hdr[BR_PH_NITEMS] = base_items;
+        hdr[BR_PH_NCOMB] = base_comb;
+        hdr[BR_PH_NONCONTIG] = s_bad;
+        hdr[BR_PH_MAX_ITEMS] = br_plan_max_items(B, M, H, T);
+        hdr[BR_PH_MAX_COMB] = br_plan_max_comb(B);
+        hdr[BR_PH_T] = T;
+    }
+}
+
+// Block table straight from per-block lengths (left- or right-aligned spans): the packed-layout
+// entry, where the caller already knows the lengths and there is no (B, M, H) mask to scan.
+__global__ void br_block_table_from_len_kernel(const int* __restrict__ lens, int BM, int H, int left_padded,
+                                               int* __restrict__ start, int* __restrict__ len) {
+    int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= BM) return;
+    int l = lens[p];
+    l = l < 0 ? 0 : (l > H ? H : l);
+    len[p] = l;
+    start[p] = left_padded ? H - l : 0;
+}
+
+}  // namespace
+
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int B, int M, int H, int T, int* plan,
+                    hipStream_t stream) {
+    int* start = plan + br_plan_off_start();
+    int* len = plan + br_plan_off_len(B, M);
+    const int BM = B * M;
+    if (valid) {
+        int waves_per_wg = 4;
+        hipLaunchKernelGGL(br_block_table_kernel, dim3((BM + waves_per_wg - 1) / waves_per_wg), dim3(256), 0, stream, valid,
+                           BM, H, start, len);
+    } else {
+        hipLaunchKernelGGL(br_block_table_from_len_kernel, dim3((BM + 255) / 256), dim3(256), 0, stream, lens, BM, H,
+                           left_padded, start, len);
+    }
+    hipLaunchKernelGGL(br_plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, plan, B, M, H, T);
+}

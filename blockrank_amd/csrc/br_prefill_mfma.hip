@@ -1,0 +1,461 @@
+// Block-sparse prefill attention for gfx950, 16-bit inputs (bf16), fp32 softmax and accumulation.
+//
+// What it computes (reference: sdpa_blockrank_attention_forward, blockrank_std_attention.py:503-650):
+// for every real query token, softmax(scale * q.k) over the keys it may see, times V, where the
+// prefix block sees itself causally, a document sees the prefix in full plus itself causally, and
+// the query block sees every earlier block in full plus itself causally.  Padded slots are neither
+// read nor written (the reference leaves an unspecified average there and never consumes it).
+//
+// How: a persistent grid pulls work items (query tile x key-walk range) from the request plan.  A
+// workgroup of NW waves stages each 64-key K tile and V^T tile in LDS once and every wave - one
+// 32-row block of one query head of the kv head's group - consumes them, so K/V are read once per
+// head group, not once per query head.  Per wave and tile:
+//   S^T = K Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q^T held in registers
+//   online softmax   each lane owns one query row and half of the tile's keys, so the row max / sum
+//                    need one cross-lane exchange (lane ^ 32) and the O rescale is a per-lane scalar
+//   O^T += V^T P^T   A = V^T rows from LDS, B = P^T straight from the S^T accumulators: the K rows
+//                    are assigned to MFMA rows in a permuted order chosen so that the accumulator
+//                    registers a lane ends up holding are exactly the 8 consecutive keys the next
+//                    MFMA's B operand wants, so P never travels through LDS.
+#include "br_common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kKPad = 8;   // bf16 elements of padding per K row in LDS
+constexpr int kVPad = 8;   // bf16 elements of padding per V^T row in LDS
+
+template <int D>
+struct Smem {
+    static constexpr int kRow = D + kKPad;                 // K tile: [64 keys][kRow]
+    static constexpr int vRow = BR_BN + kVPad;             // V^T tile: [D][vRow]
+    static constexpr int kBytes = BR_BN * kRow * 2;
+    static constexpr int vBytes = D * vRow * 2;
+    static constexpr int bufBytes = kBytes + vBytes;
+    static constexpr int eRow = D + 8;                     // epilogue tile: [32 rows][eRow] per wave
+    static constexpr int eBytesPerWave = BR_RB * eRow * 2;
+    static constexpr int total(int nw) {
+        int a = 2 * bufBytes, b = nw * eBytesPerWave;
+        return a > b ? a : b;
+    }
+};
+
+__device__ inline uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ inline bf16x8 as_bf16x8(uint4 u) {
+    union { uint4 u; bf16x8 v; } c;
+    c.u = u;
+    return c.v;
+}
+
+// Row r of a 32-row MFMA block reads key key_of_row(r) of the 32-key half tile.  With the 32x32
+// accumulator layout (lane = column + 32*h; register v is row 8*(v/4) + 4*h + v%4) this makes
+// registers 8*jp .. 8*jp+7 of lane half h hold keys 16*jp + 8*h + 0..7.
+__device__ inline int key_of_row(int r) {
+    int j = r >> 3, hr = (r >> 2) & 1, i = r & 3;
+    return 16 * (j >> 1) + 8 * hr + 4 * (j & 1) + i;
+}
+
+template <int D, int NW>
+struct Prefill {
+    static constexpr int NT = NW * 64;
+    static constexpr int CPR = D / 8;                      // 16-byte chunks per row
+    static constexpr int KCHUNKS = BR_BN * CPR;            // per K tile
+    static constexpr int KCH = (KCHUNKS + NT - 1) / NT;    // per thread
+    static constexpr int VUNITS = (BR_BN / 4) * CPR;       // 4 keys x 8 dims per unit
+    static constexpr int VCH = (VUNITS + NT - 1) / NT;
+    using SM = Smem<D>;
+
+    struct Stage {
+        uint4 k[KCH];
+        uint4 v[VCH][4];
+    };
+
+    // Issue the global loads of one K/V tile into registers.
+    static __device__ inline void load_tile(Stage& st, const BrPrefillParams& p, const __bf16* kbase, const __bf16* vbase,
+                                            int tok0, int nvalid, int tid) {
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            int ch = tid + i * NT;
+            int row = ch / CPR, c8 = ch - row * CPR;
+            uint4 z = {0u, 0u, 0u, 0u};
+            if (ch < KCHUNKS && row < nvalid) z = ld16(kbase + (long long)(tok0 + row) * p.sk_t + c8 * 8);
+            st.k[i] = z;
+        }
+#pragma unroll
+        for (int i = 0; i < VCH; ++i) {
+            int u = tid + i * NT;
+            int kq = u / CPR, dg = u - kq * CPR;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int row = kq * 4 + j;
+                uint4 z = {0u, 0u, 0u, 0u};
+                if (u < VUNITS && row < nvalid) z = ld16(vbase + (long long)(tok0 + row) * p.sv_t + dg * 8);
+                st.v[i][j] = z;
+            }
+        }
+    }
+
+    // Write the staged tile to LDS: K row-major, V transposed ([dim][key]).
+    static __device__ inline void store_tile(const Stage& st, char* buf, int tid) {
+        __bf16* Ks = reinterpret_cast<__bf16*>(buf);
+        __bf16* Vt = reinterpret_cast<__bf16*>(buf + SM::kBytes);
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            int ch = tid + i * NT;
+            int row = ch / CPR, c8 = ch - row * CPR;
+            if (ch < KCHUNKS) *reinterpret_cast<uint4*>(Ks + row * SM::kRow + c8 * 8) = st.k[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VCH; ++i) {
+            int u = tid + i * NT;
+            int kq = u / CPR, dg = u - kq * CPR;
+            if (u < VUNITS) {
+                const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&st.v[i][0]);
+                const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&st.v[i][1]);
+                const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&st.v[i][2]);
+                const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&st.v[i][3]);
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    uint2 lo, hi;   // dims 2w and 2w+1 of the unit, keys 4kq..4kq+3
+                    lo.x = (r0[w] & 0xffffu) | (r1[w] << 16);
+                    lo.y = (r2[w] & 0xffffu) | (r3[w] << 16);
+                    hi.x = (r0[w] >> 16) | (r1[w] & 0xffff0000u);
+                    hi.y = (r2[w] >> 16) | (r3[w] & 0xffff0000u);
+                    *reinterpret_cast<uint2*>(Vt + (dg * 8 + 2 * w) * SM::vRow + kq * 4) = lo;
+                    *reinterpret_cast<uint2*>(Vt + (dg * 8 + 2 * w + 1) * SM::vRow + kq * 4) = hi;
+                }
+            }
+        }
+    }
+
+    static __device__ void run_item(const BrPrefillParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem) {
+        const int tid = threadIdx.x;
+        const int wave = tid >> 6, lane = tid & 63, ln = lane & 31, lh = lane >> 5;
+        const BrGeom& ge = p.geom;
+        const int T = ge.tpb * BR_RB;
+        const int b = it.b, m = it.m;
+        const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
+        const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
+        const int head = kvh * ge.G + hsub * ge.Gw + g;
+        const int* len_b = pv.len + b * p.M;
+        const int* start_b = pv.start + b * p.M;
+        const int len_m = len_b[m];
+        const int row0 = it.t0 + sub * BR_RB;              // first query row of this wave, valid-relative
+        const bool rb_active = row0 < len_m;
+        const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
+        const int qtok0 = m * p.H + start_b[m];            // token index of the block's first real token
+
+        // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.
+        bf16x8 qf[D / 16];
+        {
+            const bool ok = row0 + ln < len_m;
+            const __bf16* qrow = reinterpret_cast<const __bf16*>(p.q) + (long long)b * p.sq_b + (long long)head * p.sq_h +
+                                 (long long)(qtok0 + row0 + ln) * p.sq_t + lh * 8;
+#pragma unroll
+            for (int c = 0; c < D / 16; ++c) {
+                uint4 z = {0u, 0u, 0u, 0u};
+                if (ok) z = ld16(qrow + c * 16);
+                qf[c] = as_bf16x8(z);
+            }
+        }
+
+        f32x16 o[D / 32];
+#pragma unroll
+        for (int d = 0; d < D / 32; ++d)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[d][v] = 0.f;
+        float m_run = -INFINITY, l_run = 0.f;
+
+        const __bf16* kbase = reinterpret_cast<const __bf16*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h;
+        const __bf16* vbase = reinterpret_cast<const __bf16*>(p.v) + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
+
+        BrWalk walk;
+        walk.init(len_b, m, p.M, self_end, it.li0, it.kt0, it.ntiles);
+        BrTile cur, nxt;
+        bool have = walk.next(cur);
+        Stage st;
+        int bufi = 0;
+        if (have) {
+            load_tile(st, p, kbase, vbase, cur.blk * p.H + start_b[cur.blk] + cur.kt * BR_BN, cur.nvalid, tid);
+            store_tile(st, smem, tid);
+        }
+        __syncthreads();
+        const int krow_off = key_of_row(ln) * SM::kRow + lh * 8;
+
+        while (have) {
+            const bool have_next = walk.next(nxt);
+            if (have_next)
+                load_tile(st, p, kbase, vbase, nxt.blk * p.H + start_b[nxt.blk] + nxt.kt * BR_BN, nxt.nvalid, tid);
+
+            const char* buf = smem + bufi * SM::bufBytes;
+            const __bf16* Ks = reinterpret_cast<const __bf16*>(buf);
+            const __bf16* Vt = reinterpret_cast<const __bf16*>(buf + SM::kBytes);
+
+            // 32-key halves of the tile this wave needs: limited by the real keys in the tile and, on
+            // the block's own keys, by the diagonal (last row of the wave is row0 + 31).
+            int nkb = (cur.nvalid + 31) >> 5;
+            const int key0 = cur.kt * BR_BN;               // valid-relative position of the tile's first key
+            if (cur.self) {
+                int vis = row0 + BR_RB - key0;             // keys [0, vis) of the tile are visible to some row
+                int c = vis <= 0 ? 0 : (vis + 31) >> 5;
+                nkb = c < nkb ? c : nkb;
+            }
+            if (!rb_active) nkb = 0;
+
+            if (nkb > 0) {
+                f32x16 s[2];
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    if (kb < nkb) {
+#pragma unroll
+                        for (int c = 0; c < D / 16; ++c) {
+                            bf16x8 a = as_bf16x8(ld16(Ks + kb * 32 * SM::kRow + krow_off + c * 16));
+                            s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], s[kb], 0, 0, 0);
+                        }
+                    }
+                }
+                // mask: keys past the tile's real keys, halves not computed, and the diagonal
+                const bool need_mask = (cur.nvalid < nkb * 32) || nkb < 2 || (cur.self && key0 + nkb * 32 - 1 > row0);
+                if (need_mask) {
+                    const int lim_valid = cur.nvalid < nkb * 32 ? cur.nvalid : nkb * 32;
+                    const int lim_causal = cur.self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
+                    const int lim = lim_valid < lim_causal ? lim_valid : lim_causal;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            int key = kb * 32 + 16 * (v >> 3) + 8 * lh + (v & 7);
+                            if (key >= lim) s[kb][v] = -INFINITY;
+                        }
+                }
+                float mx = -INFINITY;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                const float m_new = fmaxf(m_run, mx * p.scale_log2);
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+                float psum = 0.f;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        float e = __builtin_amdgcn_exp2f(s[kb][v] * p.scale_log2 - m_use);
+                        s[kb][v] = e;
+                        psum += e;
+                    }
+                m_run = m_new;
+                l_run = l_run * alpha + psum;
+#pragma unroll
+                for (int d = 0; d < D / 32; ++d)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
+
+                bf16x8 pf[4];
+#pragma unroll
+                for (int c2 = 0; c2 < 4; ++c2) {
+                    f32x8 t;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t[e] = s[c2 >> 1][8 * (c2 & 1) + e];
+                    pf[c2] = __builtin_convertvector(t, bf16x8);
+                }
+#pragma unroll
+                for (int c2 = 0; c2 < 4; ++c2) {
+                    if (c2 < 2 * nkb) {
+#pragma unroll
+                        for (int d = 0; d < D / 32; ++d) {
+                            bf16x8 a = as_bf16x8(ld16(Vt + (d * 32 + ln) * SM::vRow + c2 * 16 + lh * 8));
+                            o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[c2], o[d], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+
+            if (have_next) store_tile(st, smem + (bufi ^ 1) * SM::bufBytes, tid);
+            __syncthreads();
+            bufi ^= 1;
+            cur = nxt;
+            have = have_next;
+        }
+
+        // ---- epilogue: lane (ln, lh) holds row row0+ln, dims 32d + 8(v/4) + 4lh + v%4 ----
+        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        if (it.slot >= 0) {
+            if (row0 + ln < len_m) {
+                const long long slot = ((long long)b * BR_SLOTS_PER_SEQ + it.slot) * ge.NHG + hg;
+                const long long prow = slot * (NW * BR_RB) + wave * BR_RB + ln;
+                float* po = p.part_o + prow * D;
+#pragma unroll
+                for (int d = 0; d < D / 32; ++d)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        f32x4 t = {o[d][4 * q4], o[d][4 * q4 + 1], o[d][4 * q4 + 2], o[d][4 * q4 + 3]};
+                        *reinterpret_cast<f32x4*>(po + d * 32 + 8 * q4 + 4 * lh) = t;
+                    }
+                if (lh == 0) {
+                    p.part_ml[prow * 2] = m_run;
+                    p.part_ml[prow * 2 + 1] = l_tot;
+                }
+            }
+        } else {
+            // the last loop iteration ended with a barrier, so the K/V buffers are free: transpose
+            // through LDS so that every output row is written as full 16-byte pieces
+            __bf16* Es = reinterpret_cast<__bf16*>(smem + wave * SM::eBytesPerWave);
+            const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+            if (rb_active) {
+#pragma unroll
+                for (int d = 0; d < D / 32; ++d)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        f32x4 t = {o[d][4 * q4] * inv, o[d][4 * q4 + 1] * inv, o[d][4 * q4 + 2] * inv,
+                                   o[d][4 * q4 + 3] * inv};
+                        bf16x4 h4 = __builtin_convertvector(t, bf16x4);
+                        *reinterpret_cast<bf16x4*>(Es + ln * SM::eRow + d * 32 + 8 * q4 + 4 * lh) = h4;
+                    }
+                // same wave wrote and reads: LDS operations of one wave complete in order; the fence
+                // keeps the compiler from moving the reads above the writes
+                __threadfence_block();
+                __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
+#pragma unroll
+                for (int i = 0; i < (BR_RB * CPR) / 64; ++i) {
+                    int ch = lane + i * 64;
+                    int row = ch / CPR, c8 = ch - row * CPR;
+                    if (row0 + row < len_m) {
+                        uint4 val = ld16(Es + row * SM::eRow + c8 * 8);
+                        *reinterpret_cast<uint4*>(obase + (long long)(qtok0 + row0 + row) * p.so_t + c8 * 8) = val;
+                    }
+                }
+            }
+        }
+    }
+};
+
+template <int D, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillParams p) {
+    __shared__ __attribute__((aligned(16))) char smem[Smem<D>::total(NW)];
+    __shared__ int s_ticket;
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
+    int* hdr = const_cast<int*>(p.plan);
+    const int n_work = pv.hdr[BR_PH_NITEMS] * p.geom.NHG;
+    for (;;) {
+        if (threadIdx.x == 0) s_ticket = atomicAdd(&hdr[BR_PH_TICKET], 1);
+        __syncthreads();
+        const int w = s_ticket;
+        __syncthreads();
+        if (w >= n_work) break;
+        const int item = w / p.geom.NHG, hg = w - item * p.geom.NHG;
+        const BrItem it = pv.items[item];
+        Prefill<D, NW>::run_item(p, pv, it, hg, smem);
+    }
+    // the last workgroup to leave re-arms the counters for the next launch on this plan
+    if (threadIdx.x == 0) {
+        int d = atomicAdd(&hdr[BR_PH_DONE], 1);
+        if (d == (int)gridDim.x - 1) {
+            atomicExch(&hdr[BR_PH_TICKET], 0);
+            atomicExch(&hdr[BR_PH_DONE], 0);
+        }
+    }
+}
+
+// Merge the split-KV partials of a query tile: out = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
+template <int D>
+__global__ __launch_bounds__(256) void br_combine_kernel(BrPrefillParams p, int NW) {
+    const BrGeom& ge = p.geom;
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
+    const int n_work = pv.hdr[BR_PH_NCOMB] * ge.NHG;
+    const int m = p.M - 1;
+    for (int w = blockIdx.x; w < n_work; w += gridDim.x) {
+        const int ci = w / ge.NHG, hg = w - ci * ge.NHG;
+        const BrComb c = pv.comb[ci];
+        const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
+        const int len_m = pv.len[c.b * p.M + m];
+        const int qtok0 = m * p.H + pv.start[c.b * p.M + m];
+        const int rows = NW * BR_RB;
+        constexpr int CPR = D / 4;   // float4 chunks per row
+        for (int idx = threadIdx.x; idx < rows * CPR; idx += blockDim.x) {
+            const int r = idx / CPR, c4 = idx - r * CPR;
+            const int wave = r >> 5, n = r & 31;
+            const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
+            const int row = c.t0 + sub * BR_RB + n;
+            if (row >= len_m) continue;
+            const int head = kvh * ge.G + hsub * ge.Gw + g;
+            float mmax = -INFINITY;
+            for (int s = 0; s < c.nsplit; ++s) {
+                const long long slot = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0 + s) * ge.NHG + hg;
+                mmax = fmaxf(mmax, p.part_ml[(slot * rows + r) * 2]);
+            }
+            float l = 0.f;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < c.nsplit; ++s) {
+                const long long slot = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0 + s) * ge.NHG + hg;
+                const long long prow = slot * rows + r;
+                const float ms = p.part_ml[prow * 2];
+                const float w8 = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);
+                l += p.part_ml[prow * 2 + 1] * w8;
+                f32x4 t = *reinterpret_cast<const f32x4*>(p.part_o + prow * D + c4 * 4);
+                acc += t * w8;
+            }
+            const float inv = l > 0.f ? 1.f / l : 0.f;
+            acc *= inv;
+            bf16x4 h4 = __builtin_convertvector(acc, bf16x4);
+            __bf16* dst = reinterpret_cast<__bf16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
+                          (long long)(qtok0 + row) * p.so_t + c4 * 4;
+            *reinterpret_cast<bf16x4*>(dst) = h4;
+        }
+    }
+    // padded token slots: the kernels never touch them, so give them a defined value (zero)
+    const int n_pad_work = p.B * p.M * p.Nq;
+    for (int w = blockIdx.x; w < n_pad_work; w += gridDim.x) {
+        const int bm = w / p.Nq, head = w - bm * p.Nq;
+        const int b = bm / p.M, mm = bm - b * p.M;
+        const int st = pv.start[bm], ln = pv.len[bm];
+        const int npad = p.H - ln;
+        constexpr int CP8 = D / 8;
+        __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
+        for (int idx = threadIdx.x; idx < npad * CP8; idx += blockDim.x) {
+            int r = idx / CP8, c8 = idx - r * CP8;
+            int pos = r < st ? r : r + ln;
+            uint4 z = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<uint4*>(obase + (long long)(mm * p.H + pos) * p.so_t + c8 * 8) = z;
+        }
+    }
+}
+
+template <int D, int NW>
+void launch(const BrPrefillParams& p, int grid, hipStream_t stream) {
+    hipLaunchKernelGGL((br_prefill_mfma_kernel<D, NW>), dim3(grid), dim3(NW * 64), 0, stream, p);
+}
+
+}  // namespace
+
+// Returns 0 on success, -1 if (D, NW) has no instantiation.
+int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream) {
+    const int per_cu = NW <= 4 ? 2 : 1;
+    const int grid = n_cu * per_cu;
+#define BR_CASE(DD, WW)                                   \
+    if (D == DD && NW == WW) {                            \
+        launch<DD, WW>(p, grid, stream);                  \
+        goto launched;                                    \
+    }
+    BR_CASE(128, 4) BR_CASE(128, 5) BR_CASE(128, 6) BR_CASE(128, 7) BR_CASE(128, 8)
+    BR_CASE(64, 4) BR_CASE(64, 5) BR_CASE(64, 6) BR_CASE(64, 7) BR_CASE(64, 8)
+#undef BR_CASE
+    return -1;
+launched:
+    if (D == 128)
+        hipLaunchKernelGGL((br_combine_kernel<128>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
+    else
+        hipLaunchKernelGGL((br_combine_kernel<64>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
+    return 0;
+}

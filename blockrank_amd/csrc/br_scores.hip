@@ -1,0 +1,298 @@
+// Per-document relevance from the query block's attention, without materialising attention rows.
+//
+// Reference: compute_auxiliary_attention_loss(answer_ids=None, return_logits=True), losses.py:37-78,
+// applied to the logits of blockrank_std_attention.py:233,259 (scaled q.k of chosen rows of the
+// query block against every key).  For each (head, chosen row) the reference soft-maxes the logits
+// over all document tokens jointly and sums the probabilities per document, then averages heads and
+// rows and divides by the temperature.  Here:
+//   br_doc_partial_kernel  one workgroup per (document, kv head group, sequence): logits of that
+//                          document's real keys for every (head, row) of the group, reduced on the
+//                          fly to (max, sum of exp) per (head, row, document);
+//   br_doc_final_kernel    one workgroup per sequence: joint normalisation across documents, head /
+//                          row reduction, temperature.
+// br_last_logits_kernel writes the reference's s_last tensor itself for callers that still want it.
+#include "br_common.h"
+
+namespace {
+
+constexpr int kQR = 16;            // (head, row) pairs one workgroup carries
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T>
+struct Load8;
+template <>
+struct Load8<float> {
+    static __device__ inline void ld(const float* p, float* x) {
+        float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    }
+};
+template <>
+struct Load8<__bf16> {
+    static __device__ inline void ld(const __bf16* p, float* x) {
+        uint4 u = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[2 * i] = __uint_as_float(w[i] << 16);
+            x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
+
+struct BrScoreParams {
+    const void* q;
+    const void* k;
+    const int* plan;        // only the block table part is used
+    const int* rows;        // (B, R) positions of the chosen rows inside the query block, 0..H-1
+    float* part;            // (B, Nq, R, docs, 2): max (log2 domain) and sum of exp per document
+    float* scores;          // (B, docs)
+    float* probs;           // optional (B, Nq, R, docs) per-head, per-row document probabilities
+    float* logits;          // br_last_logits_kernel: (B, Nq, R, S)
+    long long sq_b, sq_h, sq_t;
+    long long sk_b, sk_h, sk_t;
+    int B, Nq, Nkv, M, H, D, R, T;
+    int hc;                 // heads per workgroup (hc * R <= kQR)
+    float scale;            // softmax scale
+    float out_scale;        // head/row reduction factor divided by the temperature
+    float neg;              // the reference's finite "masked" value for the model dtype
+};
+
+// Stage the (head, row) query vectors of one workgroup into LDS as fp32, pre-multiplied by mult.
+// qs is [hc*R][D]; ok[j] says whether that row is a real token.
+template <typename T>
+__device__ void stage_queries(const BrScoreParams& p, const int* start, const int* len, int b, int head0, int nheads,
+                              float mult, float* qs, int* ok) {
+    const int m = p.M - 1;
+    const int st = start[b * p.M + m], ln = len[b * p.M + m];
+    for (int idx = threadIdx.x; idx < nheads * p.R * p.D; idx += blockDim.x) {
+        int j = idx / p.D, d = idx - j * p.D;
+        int h = j / p.R, r = j - h * p.R;
+        int pos = p.rows[b * p.R + r];
+        bool v = pos >= st && pos < st + ln;
+        float x = 0.f;
+        if (v) x = (float)reinterpret_cast<const T*>(p.q)[(long long)b * p.sq_b + (long long)(head0 + h) * p.sq_h +
+                                                         (long long)(m * p.H + pos) * p.sq_t + d];
+        qs[j * p.D + d] = x * mult;
+        if (d == 0) ok[j] = v;
+    }
+}
+
+// Dot products of one key row with the nq staged query vectors.
+template <typename T>
+__device__ inline void key_dots(const T* krow, const float* qs, int nq, int D, float* s) {
+#pragma unroll
+    for (int j = 0; j < kQR; ++j) s[j] = 0.f;
+    for (int d0 = 0; d0 < D; d0 += 8) {
+        float x[8];
+        Load8<T>::ld(krow + d0, x);
+#pragma unroll
+        for (int j = 0; j < kQR; ++j) {
+            if (j < nq) {
+                const float* qv = qs + j * D + d0;
+                float a = s[j];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a = fmaf(x[e], qv[e], a);
+                s[j] = a;
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void br_doc_partial_kernel(BrScoreParams p) {
+    extern __shared__ float dyn[];
+    float* qs = dyn;                                   // [kQR][D]
+    __shared__ int ok[kQR];
+    __shared__ float red_m[4][kQR], red_s[4][kQR];
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.T);
+    const int doc = blockIdx.x, b = blockIdx.z;
+    const int G = p.Nq / p.Nkv;
+    const int chunks = (G + p.hc - 1) / p.hc;
+    const int kvh = blockIdx.y / chunks, hchunk = blockIdx.y - kvh * chunks;
+    const int head0 = kvh * G + hchunk * p.hc;
+    const int nheads = (hchunk + 1) * p.hc <= G ? p.hc : G - hchunk * p.hc;
+    const int nq = nheads * p.R;
+    const int docs = p.M - 2;
+    stage_queries<T>(p, pv.start, pv.len, b, head0, nheads, p.scale * kLog2e, qs, ok);
+    __syncthreads();
+    const int blk = doc + 1;
+    const int st = pv.start[b * p.M + blk], ln = pv.len[b * p.M + blk];
+    const T* kbase = reinterpret_cast<const T*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h +
+                     (long long)(blk * p.H + st) * p.sk_t;
+    float mx[kQR], sm[kQR];
+#pragma unroll
+    for (int j = 0; j < kQR; ++j) {
+        mx[j] = -INFINITY;
+        sm[j] = 0.f;
+    }
+    for (int key = threadIdx.x; key < ln; key += blockDim.x) {
+        float s[kQR];
+        key_dots<T>(kbase + (long long)key * p.sk_t, qs, nq, p.D, s);
+#pragma unroll
+        for (int j = 0; j < kQR; ++j) {
+            float mn = fmaxf(mx[j], s[j]);
+            sm[j] = sm[j] * __builtin_amdgcn_exp2f(mx[j] - mn) + __builtin_amdgcn_exp2f(s[j] - mn);
+            mx[j] = mn;
+        }
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int j = 0; j < kQR; ++j) {
+        float m1 = mx[j], s1 = sm[j];
+        for (int o = 32; o > 0; o >>= 1) {
+            float m2 = __shfl_xor(m1, o), s2 = __shfl_xor(s1, o);
+            float mn = fmaxf(m1, m2);
+            float a = m1 == -INFINITY ? 0.f : s1 * __builtin_amdgcn_exp2f(m1 - mn);
+            float c = m2 == -INFINITY ? 0.f : s2 * __builtin_amdgcn_exp2f(m2 - mn);
+            m1 = mn;
+            s1 = a + c;
+        }
+        if (lane == 0) {
+            red_m[wave][j] = m1;
+            red_s[wave][j] = s1;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < nq) {
+        const int j = threadIdx.x;
+        float m1 = -INFINITY, s1 = 0.f;
+        for (int w = 0; w < 4; ++w) {
+            float m2 = red_m[w][j], s2 = red_s[w][j];
+            float mn = fmaxf(m1, m2);
+            float a = m1 == -INFINITY ? 0.f : s1 * __builtin_amdgcn_exp2f(m1 - mn);
+            float c = m2 == -INFINITY ? 0.f : s2 * __builtin_amdgcn_exp2f(m2 - mn);
+            m1 = mn;
+            s1 = a + c;
+        }
+        const int h = j / p.R, r = j - h * p.R;
+        if (!ok[j]) {   // a padded query row sees nothing; the final kernel turns this into the uniform answer
+            m1 = -INFINITY;
+            s1 = 0.f;
+        }
+        float* dst = p.part + ((((long long)b * p.Nq + head0 + h) * p.R + r) * docs + doc) * 2;
+        dst[0] = m1;
+        dst[1] = s1;
+    }
+}
+
+__global__ __launch_bounds__(256) void br_doc_final_kernel(BrScoreParams p) {
+    extern __shared__ float dyn[];
+    const int NR = p.Nq * p.R;
+    const int docs = p.M - 2;
+    float* gmax = dyn;          // [NR]
+    float* ginv = dyn + NR;     // [NR], 0 marks "no visible document key": uniform
+    const int b = blockIdx.x;
+    const float* part = p.part + (long long)b * NR * docs * 2;
+    for (int j = threadIdx.x; j < NR; j += blockDim.x) {
+        float mm = -INFINITY;
+        for (int d = 0; d < docs; ++d) mm = fmaxf(mm, part[((long long)j * docs + d) * 2]);
+        float den = 0.f;
+        if (mm != -INFINITY)
+            for (int d = 0; d < docs; ++d) {
+                float m1 = part[((long long)j * docs + d) * 2];
+                if (m1 != -INFINITY) den += part[((long long)j * docs + d) * 2 + 1] * __builtin_amdgcn_exp2f(m1 - mm);
+            }
+        gmax[j] = mm;
+        ginv[j] = den > 0.f ? 1.f / den : 0.f;
+    }
+    __syncthreads();
+    const float uniform = 1.f / (float)docs;
+    for (int d = threadIdx.x; d < docs; d += blockDim.x) {
+        float acc = 0.f;
+        for (int j = 0; j < NR; ++j) {
+            float pr;
+            if (ginv[j] == 0.f) {
+                pr = uniform;
+            } else {
+                float m1 = part[((long long)j * docs + d) * 2];
+                pr = m1 == -INFINITY ? 0.f : part[((long long)j * docs + d) * 2 + 1] * __builtin_amdgcn_exp2f(m1 - gmax[j]) * ginv[j];
+            }
+            if (p.probs) p.probs[((long long)b * NR + j) * docs + d] = pr;
+            acc += pr;
+        }
+        p.scores[(long long)b * docs + d] = acc * p.out_scale;
+    }
+}
+
+// s_last[b, n, r, key] = scale * q.k + (0 if the row may see the key else NEG), every key slot of
+// the padded sequence included (blockrank_std_attention.py:639-645 with the eager scaling of :154).
+template <typename T>
+__global__ __launch_bounds__(256) void br_last_logits_kernel(BrScoreParams p) {
+    extern __shared__ float dyn[];
+    float* qs = dyn;
+    __shared__ int ok[kQR];
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.T);
+    const int b = blockIdx.z;
+    const int G = p.Nq / p.Nkv;
+    const int chunks = (G + p.hc - 1) / p.hc;
+    const int kvh = blockIdx.y / chunks, hchunk = blockIdx.y - kvh * chunks;
+    const int head0 = kvh * G + hchunk * p.hc;
+    const int nheads = (hchunk + 1) * p.hc <= G ? p.hc : G - hchunk * p.hc;
+    const int nq = nheads * p.R;
+    const int S = p.M * p.H;
+    stage_queries<T>(p, pv.start, pv.len, b, head0, nheads, p.scale, qs, ok);
+    __syncthreads();
+    const int key = blockIdx.x * blockDim.x + threadIdx.x;
+    if (key >= S) return;
+    const int blk = key / p.H, j = key - blk * p.H;
+    const int st = pv.start[b * p.M + blk], ln = pv.len[b * p.M + blk];
+    const bool kvalid = j >= st && j < st + ln;
+    const T* krow = reinterpret_cast<const T*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h + (long long)key * p.sk_t;
+    float s[kQR];
+    key_dots<T>(krow, qs, nq, p.D, s);
+#pragma unroll
+    for (int jq = 0; jq < kQR; ++jq) {
+        if (jq < nq) {
+            const int h = jq / p.R, r = jq - h * p.R;
+            const int pos = p.rows[b * p.R + r];
+            bool allow = kvalid && ok[jq] && (blk < p.M - 1 || j <= pos);
+            p.logits[(((long long)b * p.Nq + head0 + h) * p.R + r) * S + key] = s[jq] + (allow ? 0.f : p.neg);
+        }
+    }
+}
+
+}  // namespace
+
+// dtype: 0 fp32, 1 bf16
+int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
+                         float* probs, const long long* sq, const long long* sk, int B, int Nq, int Nkv, int M, int H, int D,
+                         int R, int T, float scale, float out_scale, int dtype, hipStream_t stream) {
+    BrScoreParams p;
+    p.q = q; p.k = k; p.plan = plan; p.rows = rows; p.part = part; p.scores = scores; p.probs = probs; p.logits = nullptr;
+    p.sq_b = sq[0]; p.sq_h = sq[1]; p.sq_t = sq[2];
+    p.sk_b = sk[0]; p.sk_h = sk[1]; p.sk_t = sk[2];
+    p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H; p.D = D; p.R = R; p.T = T;
+    p.hc = kQR / R; p.scale = scale; p.out_scale = out_scale; p.neg = 0.f;
+    const int G = Nq / Nkv;
+    const int chunks = (G + p.hc - 1) / p.hc;
+    dim3 grid(M - 2, Nkv * chunks, B);
+    size_t sh = (size_t)kQR * D * sizeof(float);
+    if (dtype == 0)
+        hipLaunchKernelGGL((br_doc_partial_kernel<float>), grid, dim3(256), sh, stream, p);
+    else
+        hipLaunchKernelGGL((br_doc_partial_kernel<__bf16>), grid, dim3(256), sh, stream, p);
+    hipLaunchKernelGGL(br_doc_final_kernel, dim3(B), dim3(256), (size_t)2 * Nq * R * sizeof(float), stream, p);
+    return 0;
+}
+
+int br_launch_last_logits(const void* q, const void* k, const int* plan, const int* rows, float* logits, const long long* sq,
+                          const long long* sk, int B, int Nq, int Nkv, int M, int H, int D, int R, int T, float scale,
+                          float neg, int dtype, hipStream_t stream) {
+    BrScoreParams p;
+    p.q = q; p.k = k; p.plan = plan; p.rows = rows; p.part = nullptr; p.scores = nullptr; p.probs = nullptr; p.logits = logits;
+    p.sq_b = sq[0]; p.sq_h = sq[1]; p.sq_t = sq[2];
+    p.sk_b = sk[0]; p.sk_h = sk[1]; p.sk_t = sk[2];
+    p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H; p.D = D; p.R = R; p.T = T;
+    p.hc = kQR / R; p.scale = scale; p.out_scale = 1.f; p.neg = neg;
+    const int G = Nq / Nkv;
+    const int chunks = (G + p.hc - 1) / p.hc;
+    const int S = M * H;
+    dim3 grid((S + 255) / 256, Nkv * chunks, B);
+    size_t sh = (size_t)kQR * D * sizeof(float);
+    if (dtype == 0)
+        hipLaunchKernelGGL((br_last_logits_kernel<float>), grid, dim3(256), sh, stream, p);
+    else
+        hipLaunchKernelGGL((br_last_logits_kernel<__bf16>), grid, dim3(256), sh, stream, p);
+    return 0;
+}

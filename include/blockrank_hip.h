@@ -1,0 +1,111 @@
+/* C ABI of libblockrank_hip.so: BlockRank block-sparse prefill attention and attention-score
+ * ranking on one MI355X (gfx950).
+ *
+ * The reference (nilesh2797/BlockRank) has no native layer; its path is entered through two Hugging
+ * Face registries (src/blockrank/blockrank_std_attention.py:652-665,
+ * src/blockrank/blockrank_triton_kernel_attention.py:938-965).  Each entry point below names the
+ * reference function whose work it takes over.  All pointers are device pointers unless stated;
+ * all strides are in elements; `stream` is a hipStream_t passed as void*.  Calls enqueue work on
+ * the stream and return without synchronising.  Return value 0 = success; anything else = failure,
+ * with the reason available from br_last_error() on the calling thread.
+ *
+ * Layout vocabulary: a batch of B sequences, each M blocks of H token slots (S = M*H).  Block 0 is
+ * the instruction prefix, blocks 1..M-2 the documents, block M-1 the query.  Inside a block the real
+ * tokens form one contiguous span (left padding puts it at the end of the block).
+ */
+#ifndef BLOCKRANK_HIP_H
+#define BLOCKRANK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BR_DTYPE_F32 0
+#define BR_DTYPE_BF16 1
+
+#define BR_OK 0
+#define BR_ERR_ARG 1      /* bad shape, dtype, alignment or null pointer (reference: AssertionError) */
+#define BR_ERR_SPACE 2    /* a caller-provided buffer is too small */
+#define BR_ERR_HIP 3      /* a HIP runtime call or launch failed */
+
+/* Library version, major*10000 + minor*100 + patch. */
+int br_version(void);
+
+/* Message for the last failure on this thread ("" if none). */
+const char* br_last_error(void);
+
+/* Tokens per query tile the kernels use for this head layout (the plan depends on it). 0 if the
+ * layout is unsupported (Nq not a multiple of Nkv). */
+int br_tile_tokens(int Nq, int Nkv);
+
+/* Size, in int32 elements, of the plan buffer for a (B, M, H) batch with this head layout. */
+size_t br_plan_ints(int B, int M, int H, int Nq, int Nkv);
+
+/* Build the request plan (block table + work items) from the (B, M, H) block mask, one byte per
+ * token slot, non-zero = real token.  Replaces eager_blockrank_attention_mask /
+ * triton_blockrank_attention_mask (blockrank_std_attention.py:264-309,
+ * blockrank_triton_kernel_attention.py:887-935): the 5-D additive mask those build carries exactly
+ * the per-block real-token spans, which is all the kernels need.  Build once per forward pass and
+ * pass to every layer.  One plan must not be used by two streams at the same time. */
+int br_plan_build(const uint8_t* valid, int B, int M, int H, int Nq, int Nkv, int32_t* plan, size_t plan_ints,
+                  void* stream);
+
+/* Same, from per-block real-token counts (B*M int32 on the device) instead of a mask; left_padded
+ * says at which end of its H slots each block's span sits.  No reference counterpart: it is the
+ * entry for callers that never build the padded mask
+ * (block layout of block_icr_collate_fn, src/blockrank/dataset.py:219-227). */
+int br_plan_build_from_lengths(const int32_t* lens, int left_padded, int B, int M, int H, int Nq, int Nkv,
+                               int32_t* plan, size_t plan_ints, void* stream);
+
+/* Bytes of scratch br_prefill_fwd needs (split-KV partials of the query block). */
+size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D);
+
+/* Block-sparse prefill attention.  Replaces sdpa_blockrank_attention_forward /
+ * eager_blockrank_attention_forward (blockrank_std_attention.py:472-650, :96-262) and
+ * triton_blockrank_attention_forward (blockrank_triton_kernel_attention.py:798-884) including their
+ * repeat_kv expansion and final transpose copy.
+ *   q (B, Nq, S, D), k and v (B, Nkv, S, D), out (B, Nq, S, D) logical shapes; *_strides give the
+ *   element strides of (batch, head, token); the head dimension must be dense, every stride a
+ *   multiple of 16 bytes, every base pointer 16-byte aligned.  out as the reference returns it,
+ *   (B, S, Nq, D) contiguous, is strides {S*Nq*D, D, Nq*D}.
+ *   Rows of real tokens receive the attention output; rows of padded slots are set to zero.
+ *   D in {64, 128}; dtype BR_DTYPE_BF16 (bf16 MFMA, fp32 softmax/accumulate) or BR_DTYPE_F32. */
+int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
+                   int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
+                   const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/* Bytes of scratch br_doc_scores needs. */
+size_t br_doc_scores_workspace_bytes(int B, int Nq, int M, int R);
+
+/* Fused per-document relevance.  Replaces the pair "raw logits of the last rows"
+ * (blockrank_std_attention.py:623-645; compute_last_block_attention_scores,
+ * blockrank_triton_kernel_attention.py:542-606) + compute_auxiliary_attention_loss(answer_ids=None,
+ * return_logits=True) (src/blockrank/losses.py:37-78) without materialising the logits.
+ *   rows: (B, R) int32, positions 0..H-1 inside the query block of the rows to use (the reference
+ *   uses the "[" token and the one before it); R <= 16.
+ *   scores: (B, M-2) fp32 = out_scale * sum over heads and rows of the document's probability mass
+ *   under a softmax of scale*q.k over all real document tokens.  The reference's mean over heads and
+ *   rows divided by the temperature is out_scale = 1 / (Nq * R * temperature).
+ *   probs: optional (B, Nq, R, M-2) fp32 per-head, per-row document probabilities, or NULL. */
+int br_doc_scores(const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B, int Nq,
+                  int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, float scale,
+                  float out_scale, int dtype, float* scores, float* probs, void* workspace, size_t workspace_bytes,
+                  void* stream);
+
+/* The reference's s_last tensor itself, for callers that consume it directly: logits (B, Nq, R, S)
+ * fp32 = scale * q.k + (0 where the row may see the key, else neg), for the rows given as in
+ * br_doc_scores.  Replaces blockrank_std_attention.py:242-262 / :639-645 and
+ * _compute_last_block_scores_kernel (blockrank_triton_kernel_attention.py:432-535).  neg is the
+ * reference's 0.7 * finfo(dtype).min. */
+int br_last_block_logits(const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B,
+                         int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
+                         float scale, float neg, int dtype, float* logits, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BLOCKRANK_HIP_H */
