@@ -1,0 +1,130 @@
+"""Parity of the fused per-document score kernel and of the materialised last-block logits with the
+float64 oracle.  Tolerance (from the target statement): 1e-3 relative per score, identical top-10."""
+import numpy as np
+import pytest
+import torch
+
+import blockrank_amd as br
+from blockrank_amd import synthetic
+from oracle import blockrank_oracle as orc
+from tests._util import assert_scores_close, eval_rows, oracle_doc_scores
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def fused(q, k, lay, scale, rows=None, **kw):
+    rows = eval_rows(lay, DEV) if rows is None else rows
+    return br.doc_scores(q, k, lay.valid.to(DEV), rows, scale, **kw)
+
+
+def test_config1_scores_fp32():
+    lay = synthetic.uniform_layout(1, 32, 8, 64, 16)
+    q, k, _ = synthetic.random_qkv(lay, 8, 2, 64, torch.float32, DEV)
+    got = fused(q, k, lay, 64 ** -0.5)
+    want = oracle_doc_scores(q, k, lay, 64 ** -0.5)
+    assert got.shape == (1, 8)
+    assert_scores_close(got, want)
+
+
+def test_config2_scores_bf16_full_size():
+    lay = synthetic.uniform_layout(4, 64, 20, 160, 32)
+    q, k, _ = synthetic.attention_layer_inputs(lay, 32, 8, 128, 4096, torch.bfloat16, DEV)
+    got = fused(q, k, lay, 128 ** -0.5)
+    want = oracle_doc_scores(q, k, lay, 128 ** -0.5)
+    assert got.shape == (4, 20)
+    assert_scores_close(got, want)
+    np.testing.assert_allclose(got.sum(-1).cpu().numpy() * 0.05, 1.0, rtol=1e-4)
+
+
+@pytest.mark.parametrize("Nq,Nkv,D,dtype", [(8, 2, 128, torch.bfloat16), (28, 4, 128, torch.bfloat16), (6, 2, 64, torch.float32),
+                                            (16, 1, 64, torch.bfloat16)])
+def test_ragged_documents(Nq, Nkv, D, dtype):
+    lay = synthetic.make_layout([[5, 17, 0, 300, 33, 9], [40, 1, 65, 31, 2, 70]])
+    q, k, _ = synthetic.random_qkv(lay, Nq, Nkv, D, dtype, DEV, seed=2, pad_fill=float("nan"))
+    fill = lambda t: torch.where(~lay.valid.view(lay.B, 1, lay.S, 1).to(DEV), torch.zeros_like(t), t)
+    got, probs = fused(q, k, lay, 0.11, return_probs=True)
+    want = oracle_doc_scores(fill(q), fill(k), lay, 0.11)
+    assert_scores_close(got, want)
+    assert got[0, 1].item() == 0.0                         # the empty document gets no mass
+    np.testing.assert_allclose(probs.sum(-1).cpu().numpy(), 1.0, rtol=1e-5)
+    assert probs.shape == (2, Nq, 2, 4)
+
+
+def test_training_style_rows_and_reductions():
+    # bracket not at the end (answers follow it): rows come from the labels
+    lay = synthetic.make_layout([[10, 40, 50, 24], [10, 30, 20, 24]])
+    lay.labels[:] = -100
+    lay.labels[0, -5:] = 1
+    lay.labels[1, -9:] = 1
+    q, k, _ = synthetic.random_qkv(lay, 4, 2, 64, torch.float32, DEV, seed=3)
+    h1 = 16
+    rows = torch.as_tensor(orc.bracket_rows(lay.labels.numpy(), h1)) + (lay.H - h1)
+    got = fused(q, k, lay, 0.2, rows=rows.to(DEV, torch.int32), temperature=0.1)
+    want = oracle_doc_scores(q, k, lay, 0.2, temperature=0.1, num_last=h1)
+    assert_scores_close(got, want)
+    summed = fused(q, k, lay, 0.2, rows=rows.to(DEV, torch.int32), temperature=0.1, head_reduce="sum", row_reduce="sum")
+    np.testing.assert_allclose(summed.cpu().numpy(), got.cpu().numpy() * 8, rtol=1e-6)
+
+
+def test_padded_row_gives_the_uniform_answer():
+    # a chosen row that is padding sees nothing: the reference's softmax over equal values is uniform
+    lay = synthetic.make_layout([[8, 20, 30, 40, 1]], H=48)
+    q, k, _ = synthetic.random_qkv(lay, 4, 2, 64, torch.float32, DEV, seed=4)
+    rows = torch.tensor([[lay.H - 2, lay.H - 2]], dtype=torch.int32, device=DEV)     # H-2 is padding (query has 1 token)
+    got = fused(q, k, lay, 0.3, rows=rows, temperature=1.0)
+    np.testing.assert_allclose(got.cpu().numpy(), np.full((1, 3), 1 / 3), rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_last_block_logits_match_closed_form(dtype):
+    lay = synthetic.make_layout([[9, 30, 0, 17, 20], [12, 5, 33, 8, 3]])
+    Nq, Nkv, D, R = 8, 2, 64, 16
+    q, k, _ = synthetic.random_qkv(lay, Nq, Nkv, D, dtype, DEV, seed=5)
+    rows = torch.arange(lay.H - R, lay.H, dtype=torch.int32, device=DEV)[None].expand(2, R).contiguous()
+    got = br.last_block_logits(q, k, lay.valid.to(DEV), rows, 0.17).cpu().double().numpy()
+    neg = 0.7 * torch.finfo(dtype).min
+    want = orc.last_block_logits(q.float().cpu().numpy(), k.float().cpu().numpy(), lay.valid.numpy(), 0.17, R, neg=neg)
+    assert got.shape == (2, Nq, R, lay.S)
+    ok = orc.allowed(lay.valid.numpy())[:, lay.S - R:, :]
+    okb = np.broadcast_to(ok[:, None], got.shape)
+    np.testing.assert_allclose(got[okb], want[okb], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(got[~okb], want[~okb], rtol=1e-5)      # masked: NEG plus a negligible logit
+
+
+def test_loss_api_handle_and_tensor_paths_agree():
+    lay = synthetic.uniform_layout(2, 16, 6, 48, 20)
+    Nq, Nkv, D = 8, 2, 128
+    q, k, v = synthetic.random_qkv(lay, Nq, Nkv, D, torch.bfloat16, DEV, seed=6)
+
+    class Mod:
+        layer_idx = 3
+        num_key_value_groups = 4
+        training = False
+
+    mask = br.blockrank_attention_mask(batch_size=2, attention_mask=lay.valid.to(DEV), dtype=torch.bfloat16)
+    out, h = br.blockrank_attention_forward(Mod(), q, k, v, mask, D ** -0.5, layers_to_return_scores=[3])
+    assert isinstance(h, br.LastBlockScores) and h.shape == (2, Nq, 16, lay.S)
+    _, none = br.blockrank_attention_forward(Mod(), q, k, v, mask, D ** -0.5, layers_to_return_scores=[4])
+    assert none is None
+    labels = lay.labels.to(DEV)
+    fused = br.compute_auxiliary_attention_loss(h, labels, lay.valid.to(DEV), answer_ids=None, return_logits=True)
+    dense = br.compute_auxiliary_attention_loss(h.dense(), labels, lay.valid.to(DEV), answer_ids=None, return_logits=True)
+    want = oracle_doc_scores(q, k, lay, D ** -0.5)
+    assert_scores_close(fused, want)
+    assert_scores_close(dense, want)
+    top = br.rank_documents(fused)
+    assert top.shape == (2, 6)
+    np.testing.assert_array_equal(top.cpu().numpy(), orc.topk_indices(want, 10))
+    # materialised tensor straight from the hook, and the literal-SDPA unscaled variant
+    _, t = br.blockrank_attention_forward(Mod(), q, k, v, mask, D ** -0.5, return_last_block_attn_scores=True, materialize_scores=True)
+    assert torch.is_tensor(t) and t.dtype == torch.float32 and t.shape == (2, Nq, 16, lay.S)
+    _, u = br.blockrank_attention_forward(Mod(), q, k, v, mask, D ** -0.5, return_last_block_attn_scores=True, materialize_scores=True,
+                                          unscaled_scores=True)
+    okcol = t > -1e30
+    torch.testing.assert_close(u[okcol] * D ** -0.5, t[okcol], rtol=1e-5, atol=1e-5)
+    with pytest.raises(AssertionError):
+        br.compute_auxiliary_attention_loss(h, labels, lay.valid.to(DEV), answer_ids=None, return_logits=False)
+    loss, acc, lg = br.compute_auxiliary_attention_loss(h, labels, lay.valid.to(DEV), answer_ids=torch.tensor([[0, -1], [2, 3]], device=DEV),
+                                                        return_logits=True)
+    assert torch.isfinite(loss) and 0 <= acc.item() <= 1 and torch.equal(lg, fused)
