@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the BlockRank attention + per-document score path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg4|cfg5shape|cfg1] [--no-cpu-baseline]
+
+A step is one pass of the hot path over one batch already resident in HBM: the attention hook
+(block-sparse prefill attention of one layer, query/key/value as a Mistral layer hands them over)
+followed by the fused per-document score extraction.  The request plan (block table + work items) is
+built once per forward pass by the mask hook and shared by every layer, so it is built outside the
+timed region and its cost is reported separately (``plan_build_ms``).
+
+Prints ONE JSON line: requests/s for the batch, plus
+  roofline      the main attention kernel against the bf16 MFMA peak (FLOPs of unmasked
+                (query, key) pairs only), its duration measured live with HIP events recorded
+                around the kernel on its own stream inside the timed region;
+  roofline_hbm  the same kernel against the HBM peak (algorithmic bytes: Q, K, V read once, O
+                written once) - the op sits below the machine ridge, so this roof co-binds;
+  cpu_baseline  the CPU restatement of the reference's three-call SDPA algorithm + score formula,
+                timed on this machine's host cores on a bounded sample (one sequence of the batch).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+
+
+def workloads():
+    from blockrank_amd import synthetic
+    return {
+        # BASELINE configs[1]: the configuration the headline metric is quoted on
+        "cfg2": dict(desc="Mistral-7B-shaped attention layer, B=4, 32q/8kv heads, D=128, 64-token prefix + 20 docs x 160 + 32-token query (3296 tokens/seq), bf16, proj+RoPE inputs",
+                     layout=lambda: synthetic.uniform_layout(4, 64, 20, 160, 32), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
+        # BASELINE configs[3]: long list
+        "cfg4": dict(desc="Mistral-7B attention shapes, B=1, 64-token prefix + 100 docs U[64,384] + 48-token query, bf16",
+                     layout=lambda: synthetic.random_layout(1, 64, 100, 64, 384, 48, seed=0), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
+        # BASELINE configs[4] shapes with bf16 QK^T (the fp8 variant is not built)
+        "cfg5shape": dict(desc="Qwen2.5-7B attention shapes, B=4, 28q/4kv heads, D=128, 32-token prefix + 50 lognormal docs + 24-token query, bf16",
+                          layout=lambda: synthetic.lognormal_layout(4, 32, 50, 120, 0.6, 16, 512, 24, seed=0), Nq=28, Nkv=4, D=128, hidden=3584, dtype=torch.bfloat16),
+        # BASELINE configs[0]: the reference's CPU-runnable case
+        "cfg1": dict(desc="fp32, B=1, 8q/2kv heads, D=64, 32-token prefix + 8 docs x 64 + 16-token query", layout=lambda: synthetic.uniform_layout(1, 32, 8, 64, 16),
+                     Nq=8, Nkv=2, D=64, hidden=None, dtype=torch.float32),
+    }
+
+
+class _Module:
+    """What the attention hook reads from the Hugging Face attention module."""
+    training = False
+
+    def __init__(self, layer_idx, groups):
+        self.layer_idx, self.num_key_value_groups = layer_idx, groups
+
+
+def cpu_baseline(layout, q, k, v, scale, dtype, budget_s=12.0):
+    """Time the oracle's restatement of the reference algorithm (three SDPA calls with dense additive
+    masks, GQA expansion, K0 concatenation, final transpose, 16-row logits, score formula) on the host
+    cores, for the first sequence of the batch."""
+    from oracle import blockrank_oracle as orc
+    import numpy as np
+    torch.set_num_threads(os.cpu_count() if "OMP_NUM_THREADS" not in os.environ else int(os.environ["OMP_NUM_THREADS"]))
+    q1, k1, v1 = (t[:1].detach().to("cpu", dtype).contiguous() for t in (q, k, v))
+    valid1 = layout.valid[:1]
+    labels1 = layout.labels[:1].numpy()
+    m5 = orc.additive_mask(valid1, dtype)
+
+    def one():
+        out, s_last = orc.sdpa_blockrank_forward(q1, k1, v1, m5, scale, return_scores=True)
+        return out, orc.doc_scores_from_logits(s_last.float().numpy(), labels1, valid1.numpy(), 0.05)
+
+    one()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return dict(value=1.0 / med, unit="requests/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"first sequence of the batch ({int(layout.lengths[0].sum())} tokens), {str(dtype).replace('torch.', '')}, "
+                       f"median of {len(times)} runs, {med * 1e3:.1f} ms per request",
+                ms_per_request=med * 1e3)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: ranking requests are independent and this build uses a single MI355X "
+                 "(run with --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+
+    import blockrank_amd as br
+    from blockrank_amd import profiling, synthetic
+
+    wl = workloads()[args.workload]
+    dev = torch.device("cuda:0")
+    layout = wl["layout"]()
+    Nq, Nkv, D, dtype = wl["Nq"], wl["Nkv"], wl["D"], wl["dtype"]
+    scale = D ** -0.5
+    if wl["hidden"]:
+        q, k, v = synthetic.attention_layer_inputs(layout, Nq, Nkv, D, wl["hidden"], dtype, dev)
+    else:
+        q, k, v = synthetic.random_qkv(layout, Nq, Nkv, D, dtype, dev)
+    valid = layout.valid.to(dev)
+    rows = torch.tensor([[layout.H - 2, layout.H - 1]] * layout.B, dtype=torch.int32, device=dev)   # "[" and the token before it
+    module = _Module(20, Nq // Nkv)
+
+    # once per forward pass: mask hook -> plan
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    mask = br.blockrank_attention_mask(batch_size=layout.B, attention_mask=valid, dtype=dtype)
+    mask.plan(Nq, Nkv)
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - t0) * 1e3
+
+    def step(events=None):
+        out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events)
+        scores = handle.doc_scores(rows, temperature=0.05)
+        return out, scores
+
+    for _ in range(args.warmup):
+        step()
+    pairs = [profiling.EventPair() for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        out, scores = step(pairs[i].handles)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    kern_ms = sorted(p.elapsed_ms() for p in pairs)
+    kern_avg_ms = sum(kern_ms) / len(kern_ms)
+
+    graph_ms = None
+    if args.graph:
+        g = torch.cuda.CUDAGraph()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            step()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(g, stream=s):
+                g_out, g_scores = step()
+        torch.cuda.synchronize()
+        for _ in range(5):
+            g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            g.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        assert torch.equal(g_scores, scores), "graph replay changed the scores"
+
+    pairs_n = layout.unmasked_pairs()
+    flops = 4.0 * D * pairs_n * Nq
+    esize = torch.tensor([], dtype=dtype).element_size()
+    alg_bytes = float(layout.valid_tokens) * D * esize * (2 * Nq + 2 * Nkv)
+    tflops = flops / (kern_avg_ms * 1e-3) / 1e12
+    gbs = alg_bytes / (kern_avg_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(args.workload)
+        except Exception:
+            traffic = None
+
+    best_ms = ms_per_step if graph_ms is None else min(ms_per_step, graph_ms)
+    res = {
+        "metric": "ranking requests/sec (one Mistral-7B-shaped attention layer + per-document score extraction, 20 docs)"
+        if args.workload == "cfg2" else f"ranking requests/sec ({args.workload})",
+        "value": layout.B / (best_ms * 1e-3),
+        "unit": "requests/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": best_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": wl["desc"], "name": args.workload, "batch": layout.B, "blocks": layout.M, "block_len": layout.H,
+                   "valid_tokens": layout.valid_tokens, "unmasked_pairs": pairs_n, "launch": "graph" if graph_ms is not None and graph_ms < ms_per_step else "eager"},
+        "prefill_tok_per_s": layout.valid_tokens / (best_ms * 1e-3),
+        "ms_per_step_eager": ms_per_step,
+        "ms_per_step_graph": graph_ms,
+        "plan_build_ms": plan_ms,
+        "kernel_us": {"prefill_avg": kern_avg_ms * 1e3, "prefill_p10": kern_ms[len(kern_ms) // 10] * 1e3,
+                      "prefill_p50": kern_ms[len(kern_ms) // 2] * 1e3, "prefill_p90": kern_ms[(len(kern_ms) * 9) // 10] * 1e3},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tflops / PEAK_BF16_TFLOPS,
+                     "traffic": traffic, "kernel": "br_prefill_mfma_kernel", "flops_per_launch": flops},
+        "roofline_hbm": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                         "bytes_per_launch": alg_bytes},
+    }
+    if dtype == torch.float32:
+        res["roofline"].update(bound="mfma", peak=157.3, frac=tflops / 157.3, kernel="br_prefill_f32_kernel")
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(layout, q, k, v, scale, dtype)
+        res["cpu_baseline"]["gpu_over_cpu"] = res["value"] / res["cpu_baseline"]["value"]
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -174,13 +174,16 @@ def blockrank_attention(
     value: torch.Tensor,
     block_mask,
     scaling: float,
+    *,
+    kernel_events=None,
 ) -> torch.Tensor:
     """Block-sparse prefill attention.  query (B, Nq, S, D), key/value (B, Nkv, S, D) with any
     (batch, head, token) strides; block_mask a BlockMask, a (B, M, H) bool tensor, or the reference's
     (B, 1, M, H, H) additive tensor.  Returns (B, S, Nq, D) contiguous, rows of padded slots zero.
 
     Same result as sdpa_blockrank_attention_forward (blockrank_std_attention.py:503-650) on rows of
-    real tokens."""
+    real tokens.  kernel_events: optional pair of raw hipEvent_t handles recorded right before and
+    after the main attention kernel (see blockrank_amd.profiling)."""
     if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
         block_mask = BlockMask(block_mask, query.dtype)
     bm = _as_block_mask(block_mask)
@@ -210,10 +213,11 @@ def blockrank_attention(
         ws_bytes = lib.br_prefill_workspace_bytes(B, Nq, Nkv, D)
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         out_strides = _lib._I64x3(S * Nq * D, D, Nq * D)
-        _lib.check(lib.br_prefill_fwd(
+        ev0, ev1 = kernel_events if kernel_events is not None else (None, None)
+        _lib.check(lib.br_prefill_fwd_events(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
             _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), out_strides, float(scaling), _DTYPE_CODE[query.dtype],
-            ws.data_ptr(), ws_bytes, _stream_ptr(dev)))
+            ws.data_ptr(), ws_bytes, _stream_ptr(dev), ev0, ev1))
     return out
 
 
@@ -359,7 +363,7 @@ def blockrank_attention_forward(
     if dropout > 0.0 and getattr(module, "training", False):
         warnings.warn("Dropout is not supported in kernelized BlockRank attention, ignoring dropout parameter")
 
-    out = blockrank_attention(query, key, value, bm, scaling)
+    out = blockrank_attention(query, key, value, bm, scaling, kernel_events=kwargs.get("kernel_events", None))
     if bm.M == 1:
         return out, None
 

@@ -9,8 +9,10 @@
 
 void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int B, int M, int H, int T, int* plan,
                     hipStream_t stream);
-int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream);
-int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream);
+int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
+                           hipEvent_t ev_start, hipEvent_t ev_stop);
+int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
+                           hipEvent_t ev_start, hipEvent_t ev_stop);
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
                          float* probs, const long long* sq, const long long* sk, int B, int Nq, int Nkv, int M, int H, int D,
                          int R, int T, float scale, float out_scale, int dtype, hipStream_t stream);
@@ -153,9 +155,10 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     return rows * (size_t)(D + 2) * sizeof(float);
 }
 
-int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
-                   int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                   const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                          int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                          const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
+                          void* stream, void* ev_start, void* ev_stop) {
     int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
     if (rc) return rc;
     if (!q || !k || !v || !out || !plan) return fail(BR_ERR_ARG, "null pointer");
@@ -188,10 +191,18 @@ int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const
     if (combine_grid < B * M) combine_grid = B * M;
     if (combine_grid > 4 * n_cu) combine_grid = 4 * n_cu;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    int lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s)
-                                     : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s);
+    hipEvent_t e0 = static_cast<hipEvent_t>(ev_start), e1 = static_cast<hipEvent_t>(ev_stop);
+    int lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1)
+                                     : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s, e0, e1);
     if (lrc) return fail(BR_ERR_ARG, "no kernel for head dim %d with %d query heads per kv head", D, g.G);
     return check_launch("prefill launch");
+}
+
+int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
+                   int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                   const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    return br_prefill_fwd_events(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale,
+                                 dtype, workspace, workspace_bytes, stream, nullptr, nullptr);
 }
 
 size_t br_doc_scores_workspace_bytes(int B, int Nq, int M, int R) {

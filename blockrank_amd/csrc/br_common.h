@@ -15,7 +15,7 @@
 #define BR_SLOTS_PER_SEQ 32   // split-KV partial slots available to one sequence's query block
 #define BR_MIN_CHUNK 4        // a split of the query block's key walk covers at least this many tiles
 
-// Plan buffer (int32): [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][items 8*max_items][comb 4*max_comb]
+// Plan buffer (int32): [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][items 16*max_items][comb 4*max_comb]
 #define BR_PLAN_HDR 16
 enum BrPlanHeader {
     BR_PH_NITEMS = 0,     // number of work items (per head group)
@@ -32,9 +32,14 @@ enum BrPlanHeader {
 // of its key/value tile walk.  li0/kt0 locate the first tile (walk-list position, tile inside it),
 // ntiles is how many tiles to process (INT_MAX = to the end).  slot < 0: the item owns its rows and
 // writes the final output; slot >= 0: it writes an unnormalised partial into that slot.
+// The item also carries what the kernel would otherwise have to look up in the block table before it
+// can issue its first load: the block's own span and the prefix block's span.
 struct BrItem {
-    int b, m, t0, li0, kt0, ntiles, slot, pad;
+    int b, m, t0, li0, kt0, ntiles, slot, pe;
+    int len_m, start_m, len0, start0;
+    int pad[4];
 };
+#define BR_ITEM_INTS 16
 struct BrComb {
     int b, t0, slot0, nsplit;
 };
@@ -52,7 +57,7 @@ __host__ __device__ inline size_t br_plan_off_len(int B, int M) { return BR_PLAN
 __host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M; }
 __host__ __device__ inline size_t br_plan_off_items(int B, int M) {
     size_t o = BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B;
-    return (o + 7) & ~(size_t)7;   // 32-byte aligned so an item is two 16-byte loads
+    return (o + 15) & ~(size_t)15;   // 64-byte aligned items
 }
 __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
     int qt = (H + T - 1) / T;
@@ -61,7 +66,7 @@ __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
 }
 __host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }
 __host__ __device__ inline size_t br_plan_off_comb(int B, int M, int H, int T) {
-    return br_plan_off_items(B, M) + 8 * (size_t)br_plan_max_items(B, M, H, T);
+    return br_plan_off_items(B, M) + BR_ITEM_INTS * (size_t)br_plan_max_items(B, M, H, T);
 }
 __host__ __device__ inline size_t br_plan_total_ints(int B, int M, int H, int T) {
     return br_plan_off_comb(B, M, H, T) + 4 * (size_t)br_plan_max_comb(B);
@@ -95,22 +100,23 @@ struct BrTile {
 
 struct BrWalk {
     const int* len;   // lengths of this sequence's blocks
-    int pe, m, self_end;
+    int pe, m, self_end, len0;
     int li, kt, left;
 
-    __device__ void init(const int* len_b, int m_, int M, int self_end_, int li0, int kt0, int ntiles) {
+    __device__ void init(const int* len_b, const BrItem& it, int self_end_) {
         len = len_b;
-        m = m_;
-        pe = br_prev_blocks(m_, M);
+        m = it.m;
+        pe = it.pe;
+        len0 = it.len0;
         self_end = self_end_;
-        li = li0;
-        kt = kt0;
-        left = ntiles;
+        li = it.li0;
+        kt = it.kt0;
+        left = it.ntiles;
     }
     __device__ bool next(BrTile& t) {
         if (left <= 0) return false;
         while (li <= pe) {
-            int L = li < pe ? len[li] : self_end;
+            int L = li < pe ? (li == 0 ? len0 : len[li]) : self_end;
             int k0 = kt * BR_BN;
             if (k0 < L) {
                 t.blk = li < pe ? li : m;

@@ -80,7 +80,6 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     int* prev_tiles = plan + br_plan_off_prev(B, M);
     BrItem* items = reinterpret_cast<BrItem*>(plan + br_plan_off_items(B, M));
     BrComb* comb = reinterpret_cast<BrComb*>(plan + br_plan_off_comb(B, M, H, T));
-    (void)start;
 
     if (tid < BR_PLAN_HDR) hdr[tid] = 0;
     if (tid == 0) s_bad = 0;
@@ -141,7 +140,9 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                 for (int tt = 0; tt < nq; ++tt) {
                     BrItem it;
                     it.b = b; it.m = m; it.t0 = tt * T; it.li0 = 0; it.kt0 = 0;
-                    it.ntiles = 0x7fffffff; it.slot = -1; it.pad = pe;
+                    it.ntiles = 0x7fffffff; it.slot = -1; it.pe = pe;
+                    it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
+                    it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
                     items[off_i + tt] = it;
                 }
             } else {
@@ -171,7 +172,9 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                         }
                         BrItem it;
                         it.b = b; it.m = m; it.t0 = tt * T; it.li0 = li; it.kt0 = lo - cum;
-                        it.ntiles = hi - lo; it.slot = ns > 1 ? slot + s : -1; it.pad = pe;
+                        it.ntiles = hi - lo; it.slot = ns > 1 ? slot + s : -1; it.pe = pe;
+                        it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
+                        it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
                         items[off_i++] = it;
                     }
                     if (ns > 1) slot += ns;

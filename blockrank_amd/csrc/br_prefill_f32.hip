@@ -62,7 +62,7 @@ __global__ __launch_bounds__(NW * 64) void br_prefill_f32_kernel(BrPrefillParams
         const float* vbase = V + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
 
         BrWalk walk;
-        walk.init(len_b, m, p.M, self_end, it.li0, it.kt0, it.ntiles);
+        walk.init(len_b, it, self_end);
         BrTile t;
         while (walk.next(t)) {
             const int tok0 = t.blk * p.H + start_b[t.blk] + t.kt * BR_BN;
@@ -188,8 +188,10 @@ __global__ __launch_bounds__(256) void br_combine_f32_kernel(BrPrefillParams p, 
 
 }  // namespace
 
-int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream) {
+int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
+                           hipEvent_t ev_start, hipEvent_t ev_stop) {
     const int grid = n_cu;
+    if (ev_start) (void)hipEventRecord(ev_start, stream);
 #define BR_CASE(DD, WW)                                                                                        \
     if (D == DD && NW == WW) {                                                                                 \
         hipLaunchKernelGGL((br_prefill_f32_kernel<DD, WW>), dim3(grid), dim3(WW * 64), 0, stream, p);          \
@@ -200,6 +202,7 @@ int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int
 #undef BR_CASE
     return -1;
 launched:
+    if (ev_stop) (void)hipEventRecord(ev_stop, stream);
     if (D == 128)
         hipLaunchKernelGGL((br_combine_f32_kernel<128>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
     else

@@ -4,7 +4,8 @@
 // for every real query token, softmax(scale * q.k) over the keys it may see, times V, where the
 // prefix block sees itself causally, a document sees the prefix in full plus itself causally, and
 // the query block sees every earlier block in full plus itself causally.  Padded slots are neither
-// read nor written (the reference leaves an unspecified average there and never consumes it).
+// read nor computed (the reference leaves an unspecified average there and never consumes it); the
+// finish kernel sets them to zero.
 //
 // How: a persistent grid pulls work items (query tile x key-walk range) from the request plan.  A
 // workgroup of NW waves stages each 64-key K tile and V^T tile in LDS once and every wave - one
@@ -17,6 +18,13 @@
 //                    are assigned to MFMA rows in a permuted order chosen so that the accumulator
 //                    registers a lane ends up holding are exactly the 8 consecutive keys the next
 //                    MFMA's B operand wants, so P never travels through LDS.
+//
+// LDS layouts (bank-conflict free for 16-byte reads by 8 consecutive lanes and for the transposing
+// 8-byte writes by 16 consecutive lanes):
+//   K    [64 rows][D + 8] bf16.  Row r of each 32-row half holds key swap23(r) (bits 2 and 3 of the
+//        index exchanged) so that MFMA row = LDS row and consecutive lanes read consecutive rows.
+//   V^T  [D rows][64 keys] bf16, unpadded; the 16-byte unit u (8 keys) of row d sits at unit
+//        u ^ (d & 7) ^ ((d >> 3) & 7).
 #include "br_common.h"
 
 namespace {
@@ -27,15 +35,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kKPad = 8;   // bf16 elements of padding per K row in LDS
-constexpr int kVPad = 8;   // bf16 elements of padding per V^T row in LDS
-
 template <int D>
 struct Smem {
-    static constexpr int kRow = D + kKPad;                 // K tile: [64 keys][kRow]
-    static constexpr int vRow = BR_BN + kVPad;             // V^T tile: [D][vRow]
+    static constexpr int kRow = D + 8;                     // elements per K row
     static constexpr int kBytes = BR_BN * kRow * 2;
-    static constexpr int vBytes = D * vRow * 2;
+    static constexpr int vBytes = D * BR_BN * 2;
     static constexpr int bufBytes = kBytes + vBytes;
     static constexpr int eRow = D + 8;                     // epilogue tile: [32 rows][eRow] per wave
     static constexpr int eBytesPerWave = BR_RB * eRow * 2;
@@ -51,91 +55,122 @@ __device__ inline bf16x8 as_bf16x8(uint4 u) {
     c.u = u;
     return c.v;
 }
+__device__ inline int uni(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-// Row r of a 32-row MFMA block reads key key_of_row(r) of the 32-key half tile.  With the 32x32
-// accumulator layout (lane = column + 32*h; register v is row 8*(v/4) + 4*h + v%4) this makes
-// registers 8*jp .. 8*jp+7 of lane half h hold keys 16*jp + 8*h + 0..7.
-__device__ inline int key_of_row(int r) {
-    int j = r >> 3, hr = (r >> 2) & 1, i = r & 3;
-    return 16 * (j >> 1) + 8 * hr + 4 * (j & 1) + i;
-}
+// Exchange bits 2 and 3.  MFMA row r of a 32-key half tile carries key swap23(r): with the 32x32
+// accumulator layout (lane = column + 32*h; register v is row 8*(v/4) + 4*h + v%4) registers
+// 8*jp .. 8*jp+7 of lane half h then hold keys 16*jp + 8*h + 0..7, which is the B-operand layout of
+// the P^T V product.
+__device__ inline int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
 template <int D, int NW>
 struct Prefill {
     static constexpr int NT = NW * 64;
-    static constexpr int CPR = D / 8;                      // 16-byte chunks per row
-    static constexpr int KCHUNKS = BR_BN * CPR;            // per K tile
-    static constexpr int KCH = (KCHUNKS + NT - 1) / NT;    // per thread
-    static constexpr int VUNITS = (BR_BN / 4) * CPR;       // 4 keys x 8 dims per unit
-    static constexpr int VCH = (VUNITS + NT - 1) / NT;
+    static constexpr int CPR = D / 8;                      // 16-byte chunks per K/V row
+    static constexpr int RI = NT / CPR;                    // K rows covered by one pass of the workgroup
+    static constexpr int KCH = (BR_BN + RI - 1) / RI;      // passes per K tile
+    static constexpr int VUNITS = (BR_BN / 4) * CPR;       // V staging units: 4 keys x 8 dims
     using SM = Smem<D>;
+    static_assert(VUNITS <= NT, "one V unit per thread");
+
+    // Per-thread staging constants, fixed for the whole kernel.
+    struct Lane {
+        int krow;      // K row of pass 0
+        int koff;      // element offset of this thread's K chunk inside a tile, pass 0
+        int kc8;       // chunk column
+        int vrow;      // first of the 4 V rows of this thread's unit
+        int voff;      // element offset of the unit's first row
+        int vdg, vkq;  // unit coordinates
+        bool vact;
+    };
+
+    static __device__ inline Lane make_lane(const BrPrefillParams& p, int tid) {
+        Lane L;
+        L.krow = tid / CPR;
+        L.kc8 = tid - L.krow * CPR;
+        L.koff = L.krow * (int)p.sk_t + L.kc8 * 8;
+        // V units: 16 consecutive lanes = 8 dim groups x 2 adjacent key quads, so that their 8-byte
+        // transposed writes fall into 16 different bank pairs
+        if (CPR == 16) {
+            L.vdg = (tid & 7) | (((tid >> 4) & 1) << 3);
+            L.vkq = ((tid >> 3) & 1) | ((tid >> 5) << 1);
+        } else {
+            L.vdg = tid & 7;
+            L.vkq = tid >> 3;
+        }
+        L.vact = tid < VUNITS;
+        L.vrow = L.vkq * 4;
+        L.voff = L.vrow * (int)p.sv_t + L.vdg * 8;
+        return L;
+    }
 
     struct Stage {
         uint4 k[KCH];
-        uint4 v[VCH][4];
+        uint4 v[4];
     };
 
-    // Issue the global loads of one K/V tile into registers.
-    static __device__ inline void load_tile(Stage& st, const BrPrefillParams& p, const __bf16* kbase, const __bf16* vbase,
-                                            int tok0, int nvalid, int tid) {
+    // Issue the global loads of one K/V tile into registers.  kt / vt point at the tile's first row
+    // (uniform), so every load is "uniform base + per-thread constant offset".
+    static __device__ inline void load_tile(Stage& st, const Lane& L, const __bf16* kt, const __bf16* vt, long long sk_t,
+                                            long long sv_t, int nvalid) {
+        const uint4 z = {0u, 0u, 0u, 0u};
+        if (nvalid == BR_BN) {
 #pragma unroll
-        for (int i = 0; i < KCH; ++i) {
-            int ch = tid + i * NT;
-            int row = ch / CPR, c8 = ch - row * CPR;
-            uint4 z = {0u, 0u, 0u, 0u};
-            if (ch < KCHUNKS && row < nvalid) z = ld16(kbase + (long long)(tok0 + row) * p.sk_t + c8 * 8);
-            st.k[i] = z;
-        }
+            for (int i = 0; i < KCH; ++i) {
+                if ((i + 1) * RI <= BR_BN || L.krow + i * RI < BR_BN) st.k[i] = ld16(kt + (long long)(i * RI) * sk_t + L.koff);
+            }
+            if (L.vact) {
 #pragma unroll
-        for (int i = 0; i < VCH; ++i) {
-            int u = tid + i * NT;
-            int kq = u / CPR, dg = u - kq * CPR;
+                for (int j = 0; j < 4; ++j) st.v[j] = ld16(vt + (long long)j * sv_t + L.voff);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < KCH; ++i) {
+                st.k[i] = z;
+                if (L.krow + i * RI < nvalid) st.k[i] = ld16(kt + (long long)(i * RI) * sk_t + L.koff);
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                int row = kq * 4 + j;
-                uint4 z = {0u, 0u, 0u, 0u};
-                if (u < VUNITS && row < nvalid) z = ld16(vbase + (long long)(tok0 + row) * p.sv_t + dg * 8);
-                st.v[i][j] = z;
+                st.v[j] = z;
+                if (L.vact && L.vrow + j < nvalid) st.v[j] = ld16(vt + (long long)j * sv_t + L.voff);
             }
         }
     }
 
-    // Write the staged tile to LDS: K row-major, V transposed ([dim][key]).
-    static __device__ inline void store_tile(const Stage& st, char* buf, int tid) {
+    // Write the staged tile to LDS: K rows in swap23 order, V transposed and swizzled.
+    static __device__ inline void store_tile(const Stage& st, const Lane& L, char* buf) {
         __bf16* Ks = reinterpret_cast<__bf16*>(buf);
         __bf16* Vt = reinterpret_cast<__bf16*>(buf + SM::kBytes);
 #pragma unroll
         for (int i = 0; i < KCH; ++i) {
-            int ch = tid + i * NT;
-            int row = ch / CPR, c8 = ch - row * CPR;
-            if (ch < KCHUNKS) *reinterpret_cast<uint4*>(Ks + row * SM::kRow + c8 * 8) = st.k[i];
+            const int row = L.krow + i * RI;
+            if ((i + 1) * RI <= BR_BN || row < BR_BN)
+                *reinterpret_cast<uint4*>(Ks + swap23(row) * SM::kRow + L.kc8 * 8) = st.k[i];
         }
+        if (L.vact) {
+            const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&st.v[0]);
+            const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&st.v[1]);
+            const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&st.v[2]);
+            const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&st.v[3]);
+            const int unit = L.vkq >> 1, quad = L.vkq & 1, dsw = L.vdg & 7;
 #pragma unroll
-        for (int i = 0; i < VCH; ++i) {
-            int u = tid + i * NT;
-            int kq = u / CPR, dg = u - kq * CPR;
-            if (u < VUNITS) {
-                const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&st.v[i][0]);
-                const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&st.v[i][1]);
-                const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&st.v[i][2]);
-                const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&st.v[i][3]);
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    uint2 lo, hi;   // dims 2w and 2w+1 of the unit, keys 4kq..4kq+3
-                    lo.x = (r0[w] & 0xffffu) | (r1[w] << 16);
-                    lo.y = (r2[w] & 0xffffu) | (r3[w] << 16);
-                    hi.x = (r0[w] >> 16) | (r1[w] & 0xffff0000u);
-                    hi.y = (r2[w] >> 16) | (r3[w] & 0xffff0000u);
-                    *reinterpret_cast<uint2*>(Vt + (dg * 8 + 2 * w) * SM::vRow + kq * 4) = lo;
-                    *reinterpret_cast<uint2*>(Vt + (dg * 8 + 2 * w + 1) * SM::vRow + kq * 4) = hi;
-                }
+            for (int w = 0; w < 4; ++w) {
+                uint2 lo, hi;   // dims 2w and 2w+1 of the unit, keys 4kq..4kq+3
+                lo.x = (r0[w] & 0xffffu) | (r1[w] << 16);
+                lo.y = (r2[w] & 0xffffu) | (r3[w] << 16);
+                hi.x = (r0[w] >> 16) | (r1[w] & 0xffff0000u);
+                hi.y = (r2[w] >> 16) | (r3[w] & 0xffff0000u);
+                const int d0 = L.vdg * 8 + 2 * w;
+                *reinterpret_cast<uint2*>(Vt + d0 * BR_BN + ((unit ^ dsw ^ (2 * w)) << 3) + quad * 4) = lo;
+                *reinterpret_cast<uint2*>(Vt + (d0 + 1) * BR_BN + ((unit ^ dsw ^ (2 * w + 1)) << 3) + quad * 4) = hi;
             }
         }
     }
 
-    static __device__ void run_item(const BrPrefillParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem) {
+    static __device__ void run_item(const BrPrefillParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem,
+                                    const Lane& L) {
         const int tid = threadIdx.x;
-        const int wave = tid >> 6, lane = tid & 63, ln = lane & 31, lh = lane >> 5;
+        const int wave = uni(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
         const BrGeom& ge = p.geom;
         const int T = ge.tpb * BR_RB;
         const int b = it.b, m = it.m;
@@ -144,22 +179,23 @@ struct Prefill {
         const int head = kvh * ge.G + hsub * ge.Gw + g;
         const int* len_b = pv.len + b * p.M;
         const int* start_b = pv.start + b * p.M;
-        const int len_m = len_b[m];
+        const int len_m = it.len_m;
         const int row0 = it.t0 + sub * BR_RB;              // first query row of this wave, valid-relative
         const bool rb_active = row0 < len_m;
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
-        const int qtok0 = m * p.H + start_b[m];            // token index of the block's first real token
+        const int qtok0 = m * p.H + it.start_m;            // token index of the block's first real token
 
         // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.
         bf16x8 qf[D / 16];
         {
             const bool ok = row0 + ln < len_m;
             const __bf16* qrow = reinterpret_cast<const __bf16*>(p.q) + (long long)b * p.sq_b + (long long)head * p.sq_h +
-                                 (long long)(qtok0 + row0 + ln) * p.sq_t + lh * 8;
+                                 (long long)(qtok0 + row0) * p.sq_t;
+            const int qoff = ln * (int)p.sq_t + lh * 8;
 #pragma unroll
             for (int c = 0; c < D / 16; ++c) {
                 uint4 z = {0u, 0u, 0u, 0u};
-                if (ok) z = ld16(qrow + c * 16);
+                if (ok) z = ld16(qrow + qoff + c * 16);
                 qf[c] = as_bf16x8(z);
             }
         }
@@ -175,22 +211,27 @@ struct Prefill {
         const __bf16* vbase = reinterpret_cast<const __bf16*>(p.v) + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
 
         BrWalk walk;
-        walk.init(len_b, m, p.M, self_end, it.li0, it.kt0, it.ntiles);
+        walk.init(len_b, it, self_end);
         BrTile cur, nxt;
         bool have = walk.next(cur);
         Stage st;
         int bufi = 0;
         if (have) {
-            load_tile(st, p, kbase, vbase, cur.blk * p.H + start_b[cur.blk] + cur.kt * BR_BN, cur.nvalid, tid);
-            store_tile(st, smem, tid);
+            const long long tok0 = cur.blk * p.H + (cur.blk == m ? it.start_m : (cur.blk == 0 ? it.start0 : start_b[cur.blk])) + cur.kt * BR_BN;
+            load_tile(st, L, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, p.sk_t, p.sv_t, cur.nvalid);
+            store_tile(st, L, smem);
         }
         __syncthreads();
-        const int krow_off = key_of_row(ln) * SM::kRow + lh * 8;
+        const int k_rd = ln * SM::kRow + lh * 8;                           // K operand read offset (elements)
+        const int v_rd = ln * BR_BN;                                       // V^T operand row offset
+        const int v_sw = (lh ^ (ln & 7) ^ (ln >> 3)) << 3;                 // swizzle part that depends on the lane
 
         while (have) {
             const bool have_next = walk.next(nxt);
-            if (have_next)
-                load_tile(st, p, kbase, vbase, nxt.blk * p.H + start_b[nxt.blk] + nxt.kt * BR_BN, nxt.nvalid, tid);
+            if (have_next) {
+                const long long tok0 = nxt.blk * p.H + (nxt.blk == m ? it.start_m : (nxt.blk == 0 ? it.start0 : start_b[nxt.blk])) + nxt.kt * BR_BN;
+                load_tile(st, L, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, p.sk_t, p.sv_t, nxt.nvalid);
+            }
 
             const char* buf = smem + bufi * SM::bufBytes;
             const __bf16* Ks = reinterpret_cast<const __bf16*>(buf);
@@ -218,7 +259,7 @@ struct Prefill {
                     if (kb < nkb) {
 #pragma unroll
                         for (int c = 0; c < D / 16; ++c) {
-                            bf16x8 a = as_bf16x8(ld16(Ks + kb * 32 * SM::kRow + krow_off + c * 16));
+                            bf16x8 a = as_bf16x8(ld16(Ks + kb * 32 * SM::kRow + k_rd + c * 16));
                             s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], s[kb], 0, 0, 0);
                         }
                     }
@@ -275,14 +316,15 @@ struct Prefill {
                     if (c2 < 2 * nkb) {
 #pragma unroll
                         for (int d = 0; d < D / 32; ++d) {
-                            bf16x8 a = as_bf16x8(ld16(Vt + (d * 32 + ln) * SM::vRow + c2 * 16 + lh * 8));
+                            // row 32d + ln, 16-byte unit (2*c2 + lh) ^ swizzle(row)
+                            bf16x8 a = as_bf16x8(ld16(Vt + d * 32 * BR_BN + v_rd + (v_sw ^ (((2 * c2) ^ (4 * (d & 1))) << 3))));
                             o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[c2], o[d], 0, 0, 0);
                         }
                     }
                 }
             }
 
-            if (have_next) store_tile(st, smem + (bufi ^ 1) * SM::bufBytes, tid);
+            if (have_next) store_tile(st, L, smem + (bufi ^ 1) * SM::bufBytes);
             __syncthreads();
             bufi ^= 1;
             cur = nxt;
@@ -326,14 +368,15 @@ struct Prefill {
                 // same wave wrote and reads: LDS operations of one wave complete in order; the fence
                 // keeps the compiler from moving the reads above the writes
                 __threadfence_block();
-                __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
+                __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h +
+                                (long long)(qtok0 + row0) * p.so_t;
 #pragma unroll
                 for (int i = 0; i < (BR_RB * CPR) / 64; ++i) {
                     int ch = lane + i * 64;
                     int row = ch / CPR, c8 = ch - row * CPR;
                     if (row0 + row < len_m) {
                         uint4 val = ld16(Es + row * SM::eRow + c8 * 8);
-                        *reinterpret_cast<uint4*>(obase + (long long)(qtok0 + row0 + row) * p.so_t + c8 * 8) = val;
+                        *reinterpret_cast<uint4*>(obase + row * (int)p.so_t + c8 * 8) = val;
                     }
                 }
             }
@@ -345,18 +388,25 @@ template <int D, int NW>
 __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillParams p) {
     __shared__ __attribute__((aligned(16))) char smem[Smem<D>::total(NW)];
     __shared__ int s_ticket;
+    using PF = Prefill<D, NW>;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
     const int n_work = pv.hdr[BR_PH_NITEMS] * p.geom.NHG;
+    const typename PF::Lane L = PF::make_lane(p, threadIdx.x);
+    if (threadIdx.x == 0) s_ticket = atomicAdd(&hdr[BR_PH_TICKET], 1);
+    __syncthreads();
     for (;;) {
-        if (threadIdx.x == 0) s_ticket = atomicAdd(&hdr[BR_PH_TICKET], 1);
-        __syncthreads();
-        const int w = s_ticket;
+        const int w = uni(s_ticket);
         __syncthreads();
         if (w >= n_work) break;
+        // the next ticket is fetched now and only looked at after the item: its latency is hidden
+        int next_w = 0;
+        if (threadIdx.x == 0) next_w = atomicAdd(&hdr[BR_PH_TICKET], 1);
         const int item = w / p.geom.NHG, hg = w - item * p.geom.NHG;
         const BrItem it = pv.items[item];
-        Prefill<D, NW>::run_item(p, pv, it, hg, smem);
+        PF::run_item(p, pv, it, hg, smem, L);
+        if (threadIdx.x == 0) s_ticket = next_w;
+        __syncthreads();
     }
     // the last workgroup to leave re-arms the counters for the next launch on this plan
     if (threadIdx.x == 0) {
@@ -368,50 +418,59 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     }
 }
 
-// Merge the split-KV partials of a query tile: out = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
+// Finish: (1) merge the split-KV partials of the query block,
+// out = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m); one workgroup per (query tile, head group, row
+// block); (2) set the rows of padded token slots to zero.
 template <int D>
-__global__ __launch_bounds__(256) void br_combine_kernel(BrPrefillParams p, int NW) {
+__global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int NW) {
     const BrGeom& ge = p.geom;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
-    const int n_work = pv.hdr[BR_PH_NCOMB] * ge.NHG;
+    const int n_units = pv.hdr[BR_PH_NCOMB] * ge.NHG * NW;
     const int m = p.M - 1;
-    for (int w = blockIdx.x; w < n_work; w += gridDim.x) {
+    const int rows = NW * BR_RB;
+    constexpr int CPR = D / 4;                    // float4 chunks per row
+    constexpr int TPR = 8;                        // threads per row
+    const int rr = threadIdx.x / TPR, cc = threadIdx.x % TPR;
+    for (int u = blockIdx.x; u < n_units; u += gridDim.x) {
+        const int wave = u % NW;
+        const int w = u / NW;
         const int ci = w / ge.NHG, hg = w - ci * ge.NHG;
         const BrComb c = pv.comb[ci];
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int len_m = pv.len[c.b * p.M + m];
         const int qtok0 = m * p.H + pv.start[c.b * p.M + m];
-        const int rows = NW * BR_RB;
-        constexpr int CPR = D / 4;   // float4 chunks per row
-        for (int idx = threadIdx.x; idx < rows * CPR; idx += blockDim.x) {
-            const int r = idx / CPR, c4 = idx - r * CPR;
-            const int wave = r >> 5, n = r & 31;
-            const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
-            const int row = c.t0 + sub * BR_RB + n;
-            if (row >= len_m) continue;
-            const int head = kvh * ge.G + hsub * ge.Gw + g;
-            float mmax = -INFINITY;
-            for (int s = 0; s < c.nsplit; ++s) {
-                const long long slot = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0 + s) * ge.NHG + hg;
-                mmax = fmaxf(mmax, p.part_ml[(slot * rows + r) * 2]);
-            }
-            float l = 0.f;
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            for (int s = 0; s < c.nsplit; ++s) {
-                const long long slot = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0 + s) * ge.NHG + hg;
-                const long long prow = slot * rows + r;
-                const float ms = p.part_ml[prow * 2];
-                const float w8 = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);
-                l += p.part_ml[prow * 2 + 1] * w8;
-                f32x4 t = *reinterpret_cast<const f32x4*>(p.part_o + prow * D + c4 * 4);
-                acc += t * w8;
-            }
-            const float inv = l > 0.f ? 1.f / l : 0.f;
-            acc *= inv;
-            bf16x4 h4 = __builtin_convertvector(acc, bf16x4);
-            __bf16* dst = reinterpret_cast<__bf16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
-                          (long long)(qtok0 + row) * p.so_t + c4 * 4;
-            *reinterpret_cast<bf16x4*>(dst) = h4;
+        const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
+        const int row = c.t0 + sub * BR_RB + rr;
+        if (row >= len_m) continue;
+        const int head = kvh * ge.G + hsub * ge.Gw + g;
+        const int r = wave * BR_RB + rr;
+        const long long slot0 = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0) * ge.NHG + hg;
+        const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
+        const float* ml = p.part_ml + (slot0 * rows + r) * 2;
+        float mmax = -INFINITY;
+#pragma unroll 4
+        for (int s = 0; s < c.nsplit; ++s) mmax = fmaxf(mmax, ml[s * sstride * 2]);
+        float l = 0.f;
+        f32x4 acc[CPR / TPR];
+#pragma unroll
+        for (int j = 0; j < CPR / TPR; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const float* po = p.part_o + (slot0 * rows + r) * D;
+#pragma unroll 4
+        for (int s = 0; s < c.nsplit; ++s) {
+            const float ms = ml[s * sstride * 2];
+            const float w8 = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);
+            l += ml[s * sstride * 2 + 1] * w8;
+#pragma unroll
+            for (int j = 0; j < CPR / TPR; ++j)
+                acc[j] += *reinterpret_cast<const f32x4*>(po + s * sstride * D + (cc + j * TPR) * 4) * w8;
+        }
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        __bf16* dst = reinterpret_cast<__bf16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
+                      (long long)(qtok0 + row) * p.so_t;
+#pragma unroll
+        for (int j = 0; j < CPR / TPR; ++j) {
+            bf16x4 h4 = __builtin_convertvector(acc[j] * inv, bf16x4);
+            *reinterpret_cast<bf16x4*>(dst + (cc + j * TPR) * 4) = h4;
         }
     }
     // padded token slots: the kernels never touch them, so give them a defined value (zero)
@@ -440,9 +499,11 @@ void launch(const BrPrefillParams& p, int grid, hipStream_t stream) {
 }  // namespace
 
 // Returns 0 on success, -1 if (D, NW) has no instantiation.
-int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream) {
+int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
+                           hipEvent_t ev_start, hipEvent_t ev_stop) {
     const int per_cu = NW <= 4 ? 2 : 1;
     const int grid = n_cu * per_cu;
+    if (ev_start) (void)hipEventRecord(ev_start, stream);
 #define BR_CASE(DD, WW)                                   \
     if (D == DD && NW == WW) {                            \
         launch<DD, WW>(p, grid, stream);                  \
@@ -453,9 +514,10 @@ int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, in
 #undef BR_CASE
     return -1;
 launched:
+    if (ev_stop) (void)hipEventRecord(ev_stop, stream);
     if (D == 128)
-        hipLaunchKernelGGL((br_combine_kernel<128>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
+        hipLaunchKernelGGL((br_finish_kernel<128>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
     else
-        hipLaunchKernelGGL((br_combine_kernel<64>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
+        hipLaunchKernelGGL((br_finish_kernel<64>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
     return 0;
 }

@@ -78,28 +78,32 @@ __device__ void stage_queries(const BrScoreParams& p, const int* start, const in
     }
 }
 
-// Dot products of one key row with the nq staged query vectors.
-template <typename T>
-__device__ inline void key_dots(const T* krow, const float* qs, int nq, int D, float* s) {
+// Dot products of one key row with the nq staged query vectors.  The head dim is a compile-time
+// constant so that the loop unrolls and every load of the key row is in flight before the first use.
+template <typename T, int D>
+__device__ inline void key_dots(const T* krow, const float* qs, int nq, float* s) {
 #pragma unroll
     for (int j = 0; j < kQR; ++j) s[j] = 0.f;
-    for (int d0 = 0; d0 < D; d0 += 8) {
-        float x[8];
-        Load8<T>::ld(krow + d0, x);
+    constexpr int HALF = D / 2;
+#pragma unroll
+    for (int h0 = 0; h0 < D; h0 += HALF) {
+        float x[HALF];
+#pragma unroll
+        for (int d0 = 0; d0 < HALF; d0 += 8) Load8<T>::ld(krow + h0 + d0, x + d0);
 #pragma unroll
         for (int j = 0; j < kQR; ++j) {
             if (j < nq) {
-                const float* qv = qs + j * D + d0;
+                const float* qv = qs + j * D + h0;
                 float a = s[j];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) a = fmaf(x[e], qv[e], a);
+                for (int e = 0; e < HALF; ++e) a = fmaf(x[e], qv[e], a);
                 s[j] = a;
             }
         }
     }
 }
 
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(256) void br_doc_partial_kernel(BrScoreParams p) {
     extern __shared__ float dyn[];
     float* qs = dyn;                                   // [kQR][D]
@@ -128,7 +132,7 @@ __global__ __launch_bounds__(256) void br_doc_partial_kernel(BrScoreParams p) {
     }
     for (int key = threadIdx.x; key < ln; key += blockDim.x) {
         float s[kQR];
-        key_dots<T>(kbase + (long long)key * p.sk_t, qs, nq, p.D, s);
+        key_dots<T, D>(kbase + (long long)key * p.sk_t, qs, nq, s);
 #pragma unroll
         for (int j = 0; j < kQR; ++j) {
             float mn = fmaxf(mx[j], s[j]);
@@ -184,6 +188,13 @@ __global__ __launch_bounds__(256) void br_doc_final_kernel(BrScoreParams p) {
     float* ginv = dyn + NR;     // [NR], 0 marks "no visible document key": uniform
     const int b = blockIdx.x;
     const float* part = p.part + (long long)b * NR * docs * 2;
+    // one coalesced pass brings this sequence's (max, sum) pairs into LDS when they fit
+    if (p.hc) {
+        float* stage = dyn + 2 * NR;
+        for (int i = threadIdx.x; i < NR * docs * 2; i += blockDim.x) stage[i] = part[i];
+        __syncthreads();
+        part = stage;
+    }
     for (int j = threadIdx.x; j < NR; j += blockDim.x) {
         float mm = -INFINITY;
         for (int d = 0; d < docs; ++d) mm = fmaxf(mm, part[((long long)j * docs + d) * 2]);
@@ -217,7 +228,7 @@ __global__ __launch_bounds__(256) void br_doc_final_kernel(BrScoreParams p) {
 
 // s_last[b, n, r, key] = scale * q.k + (0 if the row may see the key else NEG), every key slot of
 // the padded sequence included (blockrank_std_attention.py:639-645 with the eager scaling of :154).
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(256) void br_last_logits_kernel(BrScoreParams p) {
     extern __shared__ float dyn[];
     float* qs = dyn;
@@ -240,7 +251,7 @@ __global__ __launch_bounds__(256) void br_last_logits_kernel(BrScoreParams p) {
     const bool kvalid = j >= st && j < st + ln;
     const T* krow = reinterpret_cast<const T*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h + (long long)key * p.sk_t;
     float s[kQR];
-    key_dots<T>(krow, qs, nq, p.D, s);
+    key_dots<T, D>(krow, qs, nq, s);
 #pragma unroll
     for (int jq = 0; jq < kQR; ++jq) {
         if (jq < nq) {
@@ -268,11 +279,20 @@ int br_launch_doc_scores(const void* q, const void* k, const int* plan, const in
     const int chunks = (G + p.hc - 1) / p.hc;
     dim3 grid(M - 2, Nkv * chunks, B);
     size_t sh = (size_t)kQR * D * sizeof(float);
-    if (dtype == 0)
-        hipLaunchKernelGGL((br_doc_partial_kernel<float>), grid, dim3(256), sh, stream, p);
+    if (dtype == 0 && D == 64)
+        hipLaunchKernelGGL((br_doc_partial_kernel<float, 64>), grid, dim3(256), sh, stream, p);
+    else if (dtype == 0)
+        hipLaunchKernelGGL((br_doc_partial_kernel<float, 128>), grid, dim3(256), sh, stream, p);
+    else if (D == 64)
+        hipLaunchKernelGGL((br_doc_partial_kernel<__bf16, 64>), grid, dim3(256), sh, stream, p);
     else
-        hipLaunchKernelGGL((br_doc_partial_kernel<__bf16>), grid, dim3(256), sh, stream, p);
-    hipLaunchKernelGGL(br_doc_final_kernel, dim3(B), dim3(256), (size_t)2 * Nq * R * sizeof(float), stream, p);
+        hipLaunchKernelGGL((br_doc_partial_kernel<__bf16, 128>), grid, dim3(256), sh, stream, p);
+    // the final kernel reuses hc as "the partials fit in LDS" flag
+    size_t fin = (size_t)2 * Nq * R * sizeof(float);
+    const size_t stage = (size_t)Nq * R * (M - 2) * 2 * sizeof(float);
+    p.hc = stage + fin <= 63 * 1024 ? 1 : 0;   // stays within the default dynamic LDS limit
+    if (p.hc) fin += stage;
+    hipLaunchKernelGGL(br_doc_final_kernel, dim3(B), dim3(256), fin, stream, p);
     return 0;
 }
 
@@ -290,9 +310,13 @@ int br_launch_last_logits(const void* q, const void* k, const int* plan, const i
     const int S = M * H;
     dim3 grid((S + 255) / 256, Nkv * chunks, B);
     size_t sh = (size_t)kQR * D * sizeof(float);
-    if (dtype == 0)
-        hipLaunchKernelGGL((br_last_logits_kernel<float>), grid, dim3(256), sh, stream, p);
+    if (dtype == 0 && D == 64)
+        hipLaunchKernelGGL((br_last_logits_kernel<float, 64>), grid, dim3(256), sh, stream, p);
+    else if (dtype == 0)
+        hipLaunchKernelGGL((br_last_logits_kernel<float, 128>), grid, dim3(256), sh, stream, p);
+    else if (D == 64)
+        hipLaunchKernelGGL((br_last_logits_kernel<__bf16, 64>), grid, dim3(256), sh, stream, p);
     else
-        hipLaunchKernelGGL((br_last_logits_kernel<__bf16>), grid, dim3(256), sh, stream, p);
+        hipLaunchKernelGGL((br_last_logits_kernel<__bf16, 128>), grid, dim3(256), sh, stream, p);
     return 0;
 }

@@ -78,6 +78,14 @@ int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const
                    const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype, void* workspace,
                    size_t workspace_bytes, void* stream);
 
+/* br_prefill_fwd that also records two hipEvent_t (either may be NULL) on the stream immediately
+ * before and after the main attention kernel, so a caller can time that kernel alone inside a longer
+ * sequence of work.  No reference counterpart (the reference has no timing hooks). */
+int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
+                          int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
+                          const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype,
+                          void* workspace, size_t workspace_bytes, void* stream, void* ev_start, void* ev_stop);
+
 /* Bytes of scratch br_doc_scores needs. */
 size_t br_doc_scores_workspace_bytes(int B, int Nq, int M, int R);
 
