@@ -29,6 +29,7 @@ HIPCC_FLAGS = [
     "-fno-strict-aliasing",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",      # the LDS-DMA asm names m0 as clobbered, which clang reports as "reserved"
 ]
 
 

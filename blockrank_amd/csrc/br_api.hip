@@ -118,20 +118,25 @@ int br_tile_tokens(int Nq, int Nkv) {
 }
 
 size_t br_plan_ints(int B, int M, int H, int Nq, int Nkv) {
-    int T = br_tile_tokens(Nq, Nkv);
-    if (T == 0 || B <= 0 || M <= 0 || H <= 0) return 0;
-    return br_plan_total_ints(B, M, H, T);
+    BrGeom g;
+    int nw;
+    if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || M <= 0 || H <= 0) return 0;
+    return br_plan_total_ints(B, M, H, br_tokens_per_tile(g));
 }
 
 static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded, int B, int M, int H, int Nq, int Nkv,
                       int32_t* plan, size_t plan_ints, void* stream) {
     if (B <= 0 || M <= 0 || H <= 0) return fail(BR_ERR_ARG, "B, M and H must be positive (got %d, %d, %d)", B, M, H);
-    int T = br_tile_tokens(Nq, Nkv);
-    if (T == 0) return fail(BR_ERR_ARG, "Nq=%d must be a positive multiple of Nkv=%d", Nq, Nkv);
+    BrGeom g;
+    int nw;
+    if (!make_geom(Nq, Nkv, &g, &nw)) return fail(BR_ERR_ARG, "Nq=%d must be a positive multiple of Nkv=%d", Nq, Nkv);
+    const int T = br_tokens_per_tile(g);
     if (!plan || (!valid && !lens)) return fail(BR_ERR_ARG, "null pointer");
     if (!aligned16(plan)) return fail(BR_ERR_ARG, "plan buffer must be 16-byte aligned");
-    if (plan_ints < br_plan_total_ints(B, M, H, T))
-        return fail(BR_ERR_SPACE, "plan buffer holds %zu ints, %zu needed", plan_ints, br_plan_total_ints(B, M, H, T));
+    const size_t need = br_plan_total_ints(B, M, H, T);
+    if (plan_ints < need) return fail(BR_ERR_SPACE, "plan buffer holds %zu ints, %zu needed", plan_ints, need);
+    if ((long long)br_plan_max_items(B, M, H, T) * g.NHG >= (1 << 24))
+        return fail(BR_ERR_ARG, "batch too large for one plan (B=%d, M=%d, H=%d)", B, M, H);
     br_launch_plan(valid, lens, left_padded, B, M, H, T, plan, static_cast<hipStream_t>(stream));
     return check_launch("plan launch");
 }
@@ -232,8 +237,11 @@ int br_doc_scores(const void* q, const void* k, const int32_t* plan, const int32
     if (!workspace || workspace_bytes < need) return fail(BR_ERR_SPACE, "workspace holds %zu bytes, %zu needed", workspace_bytes, need);
     const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]};
     const long long sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
+    BrGeom g;
+    int nw;
+    make_geom(Nq, Nkv, &g, &nw);
     br_launch_doc_scores(q, k, plan, rows, static_cast<float*>(workspace), scores, probs, sq, sk, B, Nq, Nkv, M, H, D, R,
-                         br_tile_tokens(Nq, Nkv), scale, out_scale, dtype, static_cast<hipStream_t>(stream));
+                         br_tokens_per_tile(g), scale, out_scale, dtype, static_cast<hipStream_t>(stream));
     return check_launch("score launch");
 }
 
@@ -245,8 +253,11 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
     if (!logits) return fail(BR_ERR_ARG, "null pointer");
     const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]};
     const long long sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
-    br_launch_last_logits(q, k, plan, rows, logits, sq, sk, B, Nq, Nkv, M, H, D, R, br_tile_tokens(Nq, Nkv), scale, neg, dtype,
-                          static_cast<hipStream_t>(stream));
+    BrGeom g;
+    int nw;
+    make_geom(Nq, Nkv, &g, &nw);
+    br_launch_last_logits(q, k, plan, rows, logits, sq, sk, B, Nq, Nkv, M, H, D, R, br_tokens_per_tile(g), scale, neg,
+                          dtype, static_cast<hipStream_t>(stream));
     return check_launch("logits launch");
 }
 

@@ -15,17 +15,28 @@
 #define BR_SLOTS_PER_SEQ 32   // split-KV partial slots available to one sequence's query block
 #define BR_MIN_CHUNK 4        // a split of the query block's key walk covers at least this many tiles
 
-// Plan buffer (int32): [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][items 16*max_items][comb 4*max_comb]
-#define BR_PLAN_HDR 16
+// Plan buffer (int32):
+//   [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][queue lists 9*max_items]
+//   [items 16*max_items][comb 4*max_comb]
+// Work is handed out through 9 queues.  Queue 8 holds the query-block items (the long ones, with no
+// locality preference: they read every key); every workgroup drains it first.  Queues 0..7 belong
+// to the 8 XCDs: all query tiles of one (sequence, block) go to one queue, so the block's K/V for all
+// heads are fetched into one XCD's L2 only.  A ticket t of a queue is (list entry t / NHG, head group
+// t % NHG): consecutive tickets cover all kv heads, which keeps every L2 channel busy.
+#define BR_PLAN_HDR 64
+#define BR_NQUEUES 9
+#define BR_GLOBAL_QUEUE 8
 enum BrPlanHeader {
     BR_PH_NITEMS = 0,     // number of work items (per head group)
     BR_PH_NCOMB = 1,      // number of combine entries (per head group)
-    BR_PH_TICKET = 2,     // persistent-kernel ticket counter (zero between launches)
-    BR_PH_DONE = 3,       // workgroups that have left the persistent loop (zero between launches)
     BR_PH_NONCONTIG = 4,  // set to 1 if some block's real tokens are not one contiguous span
     BR_PH_MAX_ITEMS = 5,
     BR_PH_MAX_COMB = 6,
     BR_PH_T = 7,          // tokens per query tile the plan was built for
+    BR_PH_QCOUNT = 8,     // [9] items in each queue
+    // second cache line: everything the running kernels update
+    BR_PH_QTICKET = 32,   // [9] ticket counters (zero between launches)
+    BR_PH_DONE = 48,      // workgroups that have left the persistent loop (zero between launches)
 };
 
 // One unit of prefill work: query tile [t0, t0+T) of block m of sequence b, restricted to a range
@@ -46,8 +57,10 @@ struct BrComb {
 
 struct BrPlanView {
     const int* hdr;
-    const int* start;   // B*M
-    const int* len;     // B*M
+    const int* start;      // B*M
+    const int* len;        // B*M
+    const int* qlist;      // 9 lists of item indices, max_items entries apart
+    int max_items;
     const BrItem* items;
     const BrComb* comb;
 };
@@ -55,18 +68,19 @@ struct BrPlanView {
 __host__ __device__ inline size_t br_plan_off_start() { return BR_PLAN_HDR; }
 __host__ __device__ inline size_t br_plan_off_len(int B, int M) { return BR_PLAN_HDR + (size_t)B * M; }
 __host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M; }
-__host__ __device__ inline size_t br_plan_off_items(int B, int M) {
-    size_t o = BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B;
-    return (o + 15) & ~(size_t)15;   // 64-byte aligned items
-}
 __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
     int qt = (H + T - 1) / T;
     int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
     return B * ((M > 1 ? (M - 1) * qt : 0) + last);
 }
 __host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }
+__host__ __device__ inline size_t br_plan_off_qlist(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B; }
+__host__ __device__ inline size_t br_plan_off_items(int B, int M, int H, int T) {
+    size_t o = br_plan_off_qlist(B, M) + (size_t)BR_NQUEUES * br_plan_max_items(B, M, H, T);
+    return (o + 15) & ~(size_t)15;   // 64-byte aligned items
+}
 __host__ __device__ inline size_t br_plan_off_comb(int B, int M, int H, int T) {
-    return br_plan_off_items(B, M) + BR_ITEM_INTS * (size_t)br_plan_max_items(B, M, H, T);
+    return br_plan_off_items(B, M, H, T) + BR_ITEM_INTS * (size_t)br_plan_max_items(B, M, H, T);
 }
 __host__ __device__ inline size_t br_plan_total_ints(int B, int M, int H, int T) {
     return br_plan_off_comb(B, M, H, T) + 4 * (size_t)br_plan_max_comb(B);
@@ -77,9 +91,53 @@ __device__ inline BrPlanView br_plan_view(const int* plan, int B, int M, int H, 
     v.hdr = plan;
     v.start = plan + br_plan_off_start();
     v.len = plan + br_plan_off_len(B, M);
-    v.items = reinterpret_cast<const BrItem*>(plan + br_plan_off_items(B, M));
+    v.qlist = plan + br_plan_off_qlist(B, M);
+    v.max_items = br_plan_max_items(B, M, H, T);
+    v.items = reinterpret_cast<const BrItem*>(plan + br_plan_off_items(B, M, H, T));
     v.comb = reinterpret_cast<const BrComb*>(plan + br_plan_off_comb(B, M, H, T));
     return v;
+}
+
+// ---- work distribution of the persistent kernels -------------------------------------------------
+// The XCD this wave runs on (0..7).
+__device__ inline int br_xcc_id() {
+    // s_getreg_b32 HW_REG_XCC_ID (id 20), bits [3:0]
+    return __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;
+}
+
+// Queue visited at step k of a workgroup on XCD x: the global queue, its own, then the others.
+__device__ inline int br_queue_at(int k, int x) { return k == 0 ? BR_GLOBAL_QUEUE : ((x + k - 1) & 7); }
+
+// Called by one thread: take the next ticket from the queue at step *k, moving on once a queue is
+// empty (so that an XCD that runs dry helps the others).  Returns queue << 24 | ticket, or -1 when
+// every queue is exhausted.  first_ticket is a ticket already drawn from the current queue, or -1.
+__device__ inline int br_take_ticket(int* hdr, int NHG, int x, int* k, int first_ticket) {
+    int t = first_ticket;
+    while (*k < BR_NQUEUES) {
+        const int q = br_queue_at(*k, x);
+        if (t < 0) t = atomicAdd(&hdr[BR_PH_QTICKET + q], 1);
+        if (t < hdr[BR_PH_QCOUNT + q] * NHG) return (q << 24) | t;
+        ++*k;
+        t = -1;
+    }
+    return -1;
+}
+
+// Decode queue << 24 | ticket into (item index, head group).  Uniform across the workgroup.
+__device__ inline void br_decode_ticket(const BrPlanView& pv, int qt, int NHG, int& item, int& hg) {
+    const int q = qt >> 24, t = qt & 0xffffff;
+    const int li = t / NHG;
+    hg = t - li * NHG;
+    item = pv.qlist[(size_t)q * pv.max_items + li];
+}
+
+// Leave the persistent loop: the last workgroup re-arms the counters for the next launch.
+__device__ inline void br_leave(int* hdr) {
+    int d = atomicAdd(&hdr[BR_PH_DONE], 1);
+    if (d == (int)gridDim.x - 1) {
+        for (int i = 0; i < BR_NQUEUES; ++i) atomicExch(&hdr[BR_PH_QTICKET + i], 0);
+        atomicExch(&hdr[BR_PH_DONE], 0);
+    }
 }
 
 // Number of earlier blocks a query block m attends to in full: none for the prefix, the prefix for

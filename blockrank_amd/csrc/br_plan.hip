@@ -44,22 +44,26 @@ __global__ __launch_bounds__(256) void br_block_table_kernel(const uint8_t* __re
 
 __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// Exclusive scan of one int per thread over the workgroup (kPlanThreads entries); returns the
-// exclusive prefix and leaves the total in *total.
+// Exclusive scan of one int per thread over the workgroup (kPlanThreads entries): wave-level scan with
+// lane shuffles, then the 16 wave totals.  Returns the exclusive prefix, leaves the total in *total.
 __device__ int block_exclusive_scan(int x, int* sh, int* total) {
-    const int tid = threadIdx.x;
-    sh[tid] = x;
-    __syncthreads();
-    for (int o = 1; o < kPlanThreads; o <<= 1) {
-        int y = tid >= o ? sh[tid - o] : 0;
-        __syncthreads();
-        sh[tid] += y;
-        __syncthreads();
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int incl = x;
+    for (int o = 1; o < 64; o <<= 1) {
+        int y = __shfl_up(incl, o);
+        if (lane >= o) incl += y;
     }
-    int incl = sh[tid];
-    *total = sh[kPlanThreads - 1];
+    if (lane == 63) sh[wave] = incl;
     __syncthreads();
-    return incl - x;
+    int base = 0, tot = 0;
+    for (int w = 0; w < kPlanThreads / 64; ++w) {
+        int v = sh[w];
+        if (w < wave) base += v;
+        tot += v;
+    }
+    __syncthreads();
+    *total = tot;
+    return base + incl - x;
 }
 
 // Split count for query tile tt of the query block: enough splits that each covers about
@@ -71,14 +75,16 @@ __device__ inline int splits_for(int ntiles, int ns_cap) {
 }
 
 __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T) {
-    __shared__ int sh[kPlanThreads];
+    __shared__ int sh[kPlanThreads / 64];
     __shared__ int s_bad;
     const int tid = threadIdx.x;
     int* hdr = plan;
     int* start = plan + br_plan_off_start();
     int* len = plan + br_plan_off_len(B, M);
     int* prev_tiles = plan + br_plan_off_prev(B, M);
-    BrItem* items = reinterpret_cast<BrItem*>(plan + br_plan_off_items(B, M));
+    int* qlist = plan + br_plan_off_qlist(B, M);
+    const int max_items = br_plan_max_items(B, M, H, T);
+    BrItem* items = reinterpret_cast<BrItem*>(plan + br_plan_off_items(B, M, H, T));
     BrComb* comb = reinterpret_cast<BrComb*>(plan + br_plan_off_comb(B, M, H, T));
 
     if (tid < BR_PLAN_HDR) hdr[tid] = 0;
@@ -100,12 +106,14 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     }
     __syncthreads();
 
-    // Pairs are visited sequence by sequence, the query block first: its split items are the long
-    // ones and go to the front of each sequence's run of items.
+    // Pairs (sequence, block) are visited sequence by sequence, the query block first.
     int base_items = 0, base_comb = 0;
+    int qbase[BR_NQUEUES];
+#pragma unroll
+    for (int g = 0; g < BR_NQUEUES; ++g) qbase[g] = 0;
     for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
         const int p = p0 + tid;
-        int n_items = 0, n_comb = 0;
+        int n_items = 0, n_comb = 0, myq = -1;
         int b = 0, m = 0, L = 0, nq = 0, ns_cap = 1, pt = 0;
         bool is_last = false;
         if (p < BM) {
@@ -116,6 +124,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             L = len[b * M + m];
             nq = ceil_div(L, T);
             if (is_last) {
+                myq = BR_GLOBAL_QUEUE;
                 pt = M > 1 ? prev_tiles[b] : 0;
                 ns_cap = nq > 0 ? BR_SLOTS_PER_SEQ / nq : 1;
                 ns_cap = ns_cap < 1 ? 1 : ns_cap;
@@ -126,6 +135,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                     n_comb += ns > 1;
                 }
             } else {
+                myq = (b * (M - 1) + m) & 7;
                 n_items = nq;
             }
         }
@@ -134,19 +144,29 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         int off_c = base_comb + block_exclusive_scan(n_comb, sh, &tot_c);
         base_items += tot_i;
         base_comb += tot_c;
+        // position of this pair's items in its queue's list
+        int qpos = 0;
+#pragma unroll
+        for (int g = 0; g < BR_NQUEUES; ++g) {
+            int tot_g;
+            int r = block_exclusive_scan(myq == g ? n_items : 0, sh, &tot_g);
+            if (myq == g) qpos = qbase[g] + r;
+            qbase[g] += tot_g;
+        }
         if (p < BM) {
+            for (int k = 0; k < n_items; ++k) qlist[(size_t)myq * max_items + qpos + k] = off_i + k;
+            const int pe = br_prev_blocks(m, M);
+            BrItem it;
+            it.b = b; it.m = m; it.pe = pe;
+            it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
+            it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
             if (!is_last) {
-                const int pe = br_prev_blocks(m, M);
                 for (int tt = 0; tt < nq; ++tt) {
-                    BrItem it;
-                    it.b = b; it.m = m; it.t0 = tt * T; it.li0 = 0; it.kt0 = 0;
-                    it.ntiles = 0x7fffffff; it.slot = -1; it.pe = pe;
-                    it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
-                    it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
+                    it.t0 = tt * T; it.li0 = 0; it.kt0 = 0;
+                    it.ntiles = 0x7fffffff; it.slot = -1;
                     items[off_i + tt] = it;
                 }
             } else {
-                const int pe = br_prev_blocks(m, M);
                 const int* len_b = len + b * M;
                 int slot = 0;
                 for (int tt = 0; tt < nq; ++tt) {
@@ -170,11 +190,8 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                             cum += tl;
                             ++li;
                         }
-                        BrItem it;
-                        it.b = b; it.m = m; it.t0 = tt * T; it.li0 = li; it.kt0 = lo - cum;
-                        it.ntiles = hi - lo; it.slot = ns > 1 ? slot + s : -1; it.pe = pe;
-                        it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
-                        it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
+                        it.t0 = tt * T; it.li0 = li; it.kt0 = lo - cum;
+                        it.ntiles = hi - lo; it.slot = ns > 1 ? slot + s : -1;
                         items[off_i++] = it;
                     }
                     if (ns > 1) slot += ns;
@@ -184,10 +201,12 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     }
     __syncthreads();
     if (tid == 0) {
+#pragma unroll
+        for (int g = 0; g < BR_NQUEUES; ++g) hdr[BR_PH_QCOUNT + g] = qbase[g];
         hdr[BR_PH_NITEMS] = base_items;
         hdr[BR_PH_NCOMB] = base_comb;
         hdr[BR_PH_NONCONTIG] = s_bad;
-        hdr[BR_PH_MAX_ITEMS] = br_plan_max_items(B, M, H, T);
+        hdr[BR_PH_MAX_ITEMS] = max_items;
         hdr[BR_PH_MAX_COMB] = br_plan_max_comb(B);
         hdr[BR_PH_T] = T;
     }

@@ -15,26 +15,29 @@ __global__ __launch_bounds__(NW * 64) void br_prefill_f32_kernel(BrPrefillParams
     constexpr int HD = D / 2;
     __shared__ __attribute__((aligned(16))) float Ks[BR_BN * D];
     __shared__ __attribute__((aligned(16))) float Vs[BR_BN * D];
-    __shared__ int s_ticket;
+    __shared__ int s_next;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, n = lane >> 1, half = lane & 1;
     const BrGeom& ge = p.geom;
     const int T = ge.tpb * BR_RB;
+    const int NHG = ge.NHG;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, T);
     int* hdr = const_cast<int*>(p.plan);
-    const int n_work = pv.hdr[BR_PH_NITEMS] * ge.NHG;
     const float* Q = reinterpret_cast<const float*>(p.q);
     const float* K = reinterpret_cast<const float*>(p.k);
     const float* V = reinterpret_cast<const float*>(p.v);
     float* O = reinterpret_cast<float*>(p.out);
 
+    const int xcc = br_xcc_id();
+    int qk = 0;
     for (;;) {
-        if (tid == 0) s_ticket = atomicAdd(&hdr[BR_PH_TICKET], 1);
+        if (tid == 0) s_next = br_take_ticket(hdr, NHG, xcc, &qk, -1);
         __syncthreads();
-        const int w = s_ticket;
+        const int qt = __builtin_amdgcn_readfirstlane(s_next);
         __syncthreads();
-        if (w >= n_work) break;
-        const int item = w / ge.NHG, hg = w - item * ge.NHG;
+        if (qt < 0) break;
+        int item, hg;
+        br_decode_ticket(pv, qt, NHG, item, hg);
         const BrItem it = pv.items[item];
         const int b = it.b, m = it.m;
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
@@ -123,13 +126,7 @@ __global__ __launch_bounds__(NW * 64) void br_prefill_f32_kernel(BrPrefillParams
             }
         }
     }
-    if (tid == 0) {
-        int d = atomicAdd(&hdr[BR_PH_DONE], 1);
-        if (d == (int)gridDim.x - 1) {
-            atomicExch(&hdr[BR_PH_TICKET], 0);
-            atomicExch(&hdr[BR_PH_DONE], 0);
-        }
-    }
+    if (tid == 0) br_leave(hdr);
 }
 
 template <int D>

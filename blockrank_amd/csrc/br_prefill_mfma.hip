@@ -19,32 +19,38 @@
 //                    registers a lane ends up holding are exactly the 8 consecutive keys the next
 //                    MFMA's B operand wants, so P never travels through LDS.
 //
-// LDS layouts (bank-conflict free for 16-byte reads by 8 consecutive lanes and for the transposing
-// 8-byte writes by 16 consecutive lanes):
-//   K    [64 rows][D + 8] bf16.  Row r of each 32-row half holds key swap23(r) (bits 2 and 3 of the
-//        index exchanged) so that MFMA row = LDS row and consecutive lanes read consecutive rows.
-//   V^T  [D rows][64 keys] bf16, unpadded; the 16-byte unit u (8 keys) of row d sits at unit
-//        u ^ (d & 7) ^ ((d >> 3) & 7).
+// Data movement: K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4, 64
+// lanes x 16 bytes per instruction, no staging registers); which 16-byte piece of which row a lane
+// fetches is free, and that freedom provides both the row permutation and the swizzles below.  V is
+// kept row-major ([key][dim]) and read with ds_read_b64_tr_b16, which hands each lane four
+// consecutive keys of one dim - the MFMA A-operand layout of V^T - so V is never transposed by ALU code.
+//
+// LDS layouts (row = 2*D bytes, 16-byte chunks; reads are bank-conflict free):
+//   K    row r of each 32-row half holds key swap23(r) (bits 2 and 3 of the index exchanged) so that
+//        MFMA row = LDS row; chunk c of row r sits at chunk c ^ (r & 7).
+//   V    row = key; chunk c of row r sits at chunk c ^ ((r & 3) << 1).
 #include "br_common.h"
 
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 template <int D>
 struct Smem {
-    static constexpr int kRow = D + 8;                     // elements per K row
-    static constexpr int kBytes = BR_BN * kRow * 2;
-    static constexpr int vBytes = D * BR_BN * 2;
-    static constexpr int bufBytes = kBytes + vBytes;
+    static constexpr int rowB = D * 2;                     // bytes per K or V row
+    static constexpr int kBytes = BR_BN * rowB;
+    static constexpr int stageBytes = 2 * kBytes;          // K tile then V tile
     static constexpr int eRow = D + 8;                     // epilogue tile: [32 rows][eRow] per wave
     static constexpr int eBytesPerWave = BR_RB * eRow * 2;
     static constexpr int total(int nw) {
-        int a = 2 * bufBytes, b = nw * eBytesPerWave;
+        int a = 2 * stageBytes, b = nw * eBytesPerWave;
         return a > b ? a : b;
     }
 };
@@ -57,6 +63,18 @@ __device__ inline bf16x8 as_bf16x8(uint4 u) {
 }
 __device__ inline int uni(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
+// 64 lanes x 16 bytes from global memory (uniform base + per-lane byte offset) into LDS at
+// lds_addr + lane * 16.  Issued through asm so that the compiler does not make later LDS reads of
+// other buffers wait for it; completion is awaited explicitly (vm_wait_all) before the barrier that
+// publishes the tile.
+__device__ inline void dma16(const void* base, int byte_off, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+__device__ inline void vm_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ inline unsigned lds_addr_of(const void* p) {
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const void*)p;
+}
+
 // Exchange bits 2 and 3.  MFMA row r of a 32-key half tile carries key swap23(r): with the 32x32
 // accumulator layout (lane = column + 32*h; register v is row 8*(v/4) + 4*h + v%4) registers
 // 8*jp .. 8*jp+7 of lane half h then hold keys 16*jp + 8*h + 0..7, which is the B-operand layout of
@@ -65,104 +83,62 @@ __device__ inline int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 
 
 template <int D, int NW>
 struct Prefill {
-    static constexpr int NT = NW * 64;
     static constexpr int CPR = D / 8;                      // 16-byte chunks per K/V row
-    static constexpr int RI = NT / CPR;                    // K rows covered by one pass of the workgroup
-    static constexpr int KCH = (BR_BN + RI - 1) / RI;      // passes per K tile
-    static constexpr int VUNITS = (BR_BN / 4) * CPR;       // V staging units: 4 keys x 8 dims
+    static constexpr int NI = BR_BN * CPR / 64;            // DMA instructions per K (or V) tile
+    static constexpr int JK = (NI + NW - 1) / NW;          // per wave
     using SM = Smem<D>;
-    static_assert(VUNITS <= NT, "one V unit per thread");
 
-    // Per-thread staging constants, fixed for the whole kernel.
+    // Per-lane constants, fixed for the whole kernel.
     struct Lane {
-        int krow;      // K row of pass 0
-        int koff;      // element offset of this thread's K chunk inside a tile, pass 0
-        int kc8;       // chunk column
-        int vrow;      // first of the 4 V rows of this thread's unit
-        int voff;      // element offset of the unit's first row
-        int vdg, vkq;  // unit coordinates
-        bool vact;
+        int koff[JK], voff[JK];    // global byte offsets inside a tile of this lane's DMA pieces
+        int krd[D / 16];           // LDS byte offsets of the K operand reads, one per 16-dim chunk
+        int vrd[D / 32];           // LDS byte offsets of the V^T operand reads, one per 32-dim block
     };
 
-    static __device__ inline Lane make_lane(const BrPrefillParams& p, int tid) {
+    static __device__ inline Lane make_lane(const BrPrefillParams& p, int wave, int lane) {
         Lane L;
-        L.krow = tid / CPR;
-        L.kc8 = tid - L.krow * CPR;
-        L.koff = L.krow * (int)p.sk_t + L.kc8 * 8;
-        // V units: 16 consecutive lanes = 8 dim groups x 2 adjacent key quads, so that their 8-byte
-        // transposed writes fall into 16 different bank pairs
-        if (CPR == 16) {
-            L.vdg = (tid & 7) | (((tid >> 4) & 1) << 3);
-            L.vkq = ((tid >> 3) & 1) | ((tid >> 5) << 1);
-        } else {
-            L.vdg = tid & 7;
-            L.vkq = tid >> 3;
+#pragma unroll
+        for (int j = 0; j < JK; ++j) {
+            const int slot = (wave + NW * j) * 64 + lane;
+            const int prow = slot / CPR, cp = slot - prow * CPR;
+            const int kkey = (prow & 32) | swap23(prow & 31);
+            L.koff[j] = kkey * (int)p.sk_t * 2 + ((cp ^ (prow & 7)) << 4);
+            L.voff[j] = prow * (int)p.sv_t * 2 + ((cp ^ ((prow & 3) << 1)) << 4);
         }
-        L.vact = tid < VUNITS;
-        L.vrow = L.vkq * 4;
-        L.voff = L.vrow * (int)p.sv_t + L.vdg * 8;
+        const int ln = lane & 31, lh = lane >> 5;
+#pragma unroll
+        for (int c = 0; c < D / 16; ++c) L.krd[c] = ln * SM::rowB + (((2 * c + lh) ^ (ln & 7)) << 4);
+        // transposing read: within a group of 16 lanes, lane s points at key (s >> 2), dims 4 * (s & 3)
+        const int s = lane & 15, ln_hi = (lane >> 4) & 1;
+        const int cl = (2 * ln_hi + ((s & 3) >> 1)) ^ ((s >> 2) << 1);
+#pragma unroll
+        for (int d = 0; d < D / 32; ++d)
+            L.vrd[d] = SM::kBytes + (8 * lh + (s >> 2)) * SM::rowB + (((4 * d) ^ cl) << 4) + (s & 1) * 8;
         return L;
     }
 
-    struct Stage {
-        uint4 k[KCH];
-        uint4 v[4];
-    };
-
-    // Issue the global loads of one K/V tile into registers.  kt / vt point at the tile's first row
-    // (uniform), so every load is "uniform base + per-thread constant offset".
-    static __device__ inline void load_tile(Stage& st, const Lane& L, const __bf16* kt, const __bf16* vt, long long sk_t,
-                                            long long sv_t, int nvalid) {
-        const uint4 z = {0u, 0u, 0u, 0u};
+    // Start the DMA of one K/V tile into a stage.  kt / vt point at the tile's first row (uniform).
+    static __device__ inline void issue_tile(const Lane& L, int wave, const __bf16* kt, const __bf16* vt, int sk_bytes, int sv_bytes,
+                                             int nvalid, unsigned stage_lds) {
         if (nvalid == BR_BN) {
 #pragma unroll
-            for (int i = 0; i < KCH; ++i) {
-                if ((i + 1) * RI <= BR_BN || L.krow + i * RI < BR_BN) st.k[i] = ld16(kt + (long long)(i * RI) * sk_t + L.koff);
-            }
-            if (L.vact) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) st.v[j] = ld16(vt + (long long)j * sv_t + L.voff);
+            for (int j = 0; j < JK; ++j) {
+                const int q = wave + NW * j;
+                if (NI % NW == 0 || q < NI) {
+                    dma16(kt, L.koff[j], stage_lds + q * 1024);
+                    dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
+                }
             }
         } else {
+            // rows past the tile's real keys are not fetched: the LDS rows keep older (finite) data,
+            // which the kernel masks (K) or multiplies by exact zeros (V)
 #pragma unroll
-            for (int i = 0; i < KCH; ++i) {
-                st.k[i] = z;
-                if (L.krow + i * RI < nvalid) st.k[i] = ld16(kt + (long long)(i * RI) * sk_t + L.koff);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                st.v[j] = z;
-                if (L.vact && L.vrow + j < nvalid) st.v[j] = ld16(vt + (long long)j * sv_t + L.voff);
-            }
-        }
-    }
-
-    // Write the staged tile to LDS: K rows in swap23 order, V transposed and swizzled.
-    static __device__ inline void store_tile(const Stage& st, const Lane& L, char* buf) {
-        __bf16* Ks = reinterpret_cast<__bf16*>(buf);
-        __bf16* Vt = reinterpret_cast<__bf16*>(buf + SM::kBytes);
-#pragma unroll
-        for (int i = 0; i < KCH; ++i) {
-            const int row = L.krow + i * RI;
-            if ((i + 1) * RI <= BR_BN || row < BR_BN)
-                *reinterpret_cast<uint4*>(Ks + swap23(row) * SM::kRow + L.kc8 * 8) = st.k[i];
-        }
-        if (L.vact) {
-            const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&st.v[0]);
-            const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&st.v[1]);
-            const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&st.v[2]);
-            const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&st.v[3]);
-            const int unit = L.vkq >> 1, quad = L.vkq & 1, dsw = L.vdg & 7;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                uint2 lo, hi;   // dims 2w and 2w+1 of the unit, keys 4kq..4kq+3
-                lo.x = (r0[w] & 0xffffu) | (r1[w] << 16);
-                lo.y = (r2[w] & 0xffffu) | (r3[w] << 16);
-                hi.x = (r0[w] >> 16) | (r1[w] & 0xffff0000u);
-                hi.y = (r2[w] >> 16) | (r3[w] & 0xffff0000u);
-                const int d0 = L.vdg * 8 + 2 * w;
-                *reinterpret_cast<uint2*>(Vt + d0 * BR_BN + ((unit ^ dsw ^ (2 * w)) << 3) + quad * 4) = lo;
-                *reinterpret_cast<uint2*>(Vt + (d0 + 1) * BR_BN + ((unit ^ dsw ^ (2 * w + 1)) << 3) + quad * 4) = hi;
+            for (int j = 0; j < JK; ++j) {
+                const int q = wave + NW * j;
+                if (NI % NW == 0 || q < NI) {
+                    if (L.koff[j] < nvalid * sk_bytes) dma16(kt, L.koff[j], stage_lds + q * 1024);
+                    if (L.voff[j] < nvalid * sv_bytes) dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
+                }
             }
         }
     }
@@ -184,6 +160,20 @@ struct Prefill {
         const bool rb_active = row0 < len_m;
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
         const int qtok0 = m * p.H + it.start_m;            // token index of the block's first real token
+        const unsigned smem_lds = lds_addr_of(smem);
+        const int sk_bytes = (int)p.sk_t * 2, sv_bytes = (int)p.sv_t * 2;
+
+        const __bf16* kbase = reinterpret_cast<const __bf16*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h;
+        const __bf16* vbase = reinterpret_cast<const __bf16*>(p.v) + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
+
+        BrWalk walk;
+        walk.init(len_b, it, self_end);
+        BrTile cur, nxt;
+        bool have = walk.next(cur);
+        if (have) {
+            const long long tok0 = cur.blk * p.H + (cur.blk == m ? it.start_m : (cur.blk == 0 ? it.start0 : start_b[cur.blk])) + cur.kt * BR_BN;
+            issue_tile(L, wave, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, sk_bytes, sv_bytes, cur.nvalid, smem_lds);
+        }
 
         // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.
         bf16x8 qf[D / 16];
@@ -207,35 +197,18 @@ struct Prefill {
             for (int v = 0; v < 16; ++v) o[d][v] = 0.f;
         float m_run = -INFINITY, l_run = 0.f;
 
-        const __bf16* kbase = reinterpret_cast<const __bf16*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h;
-        const __bf16* vbase = reinterpret_cast<const __bf16*>(p.v) + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
-
-        BrWalk walk;
-        walk.init(len_b, it, self_end);
-        BrTile cur, nxt;
-        bool have = walk.next(cur);
-        Stage st;
-        int bufi = 0;
-        if (have) {
-            const long long tok0 = cur.blk * p.H + (cur.blk == m ? it.start_m : (cur.blk == 0 ? it.start0 : start_b[cur.blk])) + cur.kt * BR_BN;
-            load_tile(st, L, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, p.sk_t, p.sv_t, cur.nvalid);
-            store_tile(st, L, smem);
-        }
+        vm_wait_all();
         __syncthreads();
-        const int k_rd = ln * SM::kRow + lh * 8;                           // K operand read offset (elements)
-        const int v_rd = ln * BR_BN;                                       // V^T operand row offset
-        const int v_sw = (lh ^ (ln & 7) ^ (ln >> 3)) << 3;                 // swizzle part that depends on the lane
+        int bufi = 0;
 
         while (have) {
             const bool have_next = walk.next(nxt);
             if (have_next) {
                 const long long tok0 = nxt.blk * p.H + (nxt.blk == m ? it.start_m : (nxt.blk == 0 ? it.start0 : start_b[nxt.blk])) + nxt.kt * BR_BN;
-                load_tile(st, L, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, p.sk_t, p.sv_t, nxt.nvalid);
+                issue_tile(L, wave, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, sk_bytes, sv_bytes, nxt.nvalid,
+                           smem_lds + (bufi ^ 1) * SM::stageBytes);
             }
-
-            const char* buf = smem + bufi * SM::bufBytes;
-            const __bf16* Ks = reinterpret_cast<const __bf16*>(buf);
-            const __bf16* Vt = reinterpret_cast<const __bf16*>(buf + SM::kBytes);
+            const char* stage = smem + bufi * SM::stageBytes;
 
             // 32-key halves of the tile this wave needs: limited by the real keys in the tile and, on
             // the block's own keys, by the diagonal (last row of the wave is row0 + 31).
@@ -250,26 +223,27 @@ struct Prefill {
 
             if (nkb > 0) {
                 f32x16 s[2];
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) {
                     if (kb < nkb) {
+                        f32x16 acc = zero;
 #pragma unroll
                         for (int c = 0; c < D / 16; ++c) {
-                            bf16x8 a = as_bf16x8(ld16(Ks + kb * 32 * SM::kRow + k_rd + c * 16));
-                            s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], s[kb], 0, 0, 0);
+                            bf16x8 a = as_bf16x8(ld16(stage + kb * 32 * SM::rowB + L.krd[c]));
+                            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], acc, 0, 0, 0);
                         }
+                        s[kb] = acc;
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) s[kb][v] = -INFINITY;
                     }
                 }
-                // mask: keys past the tile's real keys, halves not computed, and the diagonal
-                const bool need_mask = (cur.nvalid < nkb * 32) || nkb < 2 || (cur.self && key0 + nkb * 32 - 1 > row0);
+                // mask keys past the tile's real keys and beyond the diagonal
+                const bool need_mask = (cur.nvalid < nkb * 32) || (cur.self && key0 + nkb * 32 - 1 > row0);
                 if (need_mask) {
-                    const int lim_valid = cur.nvalid < nkb * 32 ? cur.nvalid : nkb * 32;
                     const int lim_causal = cur.self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
-                    const int lim = lim_valid < lim_causal ? lim_valid : lim_causal;
+                    const int lim = cur.nvalid < lim_causal ? cur.nvalid : lim_causal;
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -284,24 +258,31 @@ struct Prefill {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
                 mx = fmaxf(mx, __shfl_xor(mx, 32));
+                // Lazy rescale: the running max is only raised (and O, l rescaled) when some row's max
+                // grew by more than 2^8; otherwise exponentials are taken against the older max, which
+                // changes nothing in the final quotient and keeps them below 2^8.
                 const float m_new = fmaxf(m_run, mx * p.scale_log2);
-                const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+                if (__builtin_amdgcn_ballot_w64(m_new - m_run > 8.f) != 0) {
+                    const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+                    const float alpha = __builtin_amdgcn_exp2f(m_run - m_sub);
+                    m_run = m_new;
+                    l_run *= alpha;
+#pragma unroll
+                    for (int d = 0; d < D / 32; ++d)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
+                }
+                const float m_sub = m_run == -INFINITY ? 0.f : m_run;
                 float psum = 0.f;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
-                        float e = __builtin_amdgcn_exp2f(s[kb][v] * p.scale_log2 - m_use);
+                        float e = __builtin_amdgcn_exp2f(s[kb][v] * p.scale_log2 - m_sub);
                         s[kb][v] = e;
                         psum += e;
                     }
-                m_run = m_new;
-                l_run = l_run * alpha + psum;
-#pragma unroll
-                for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
+                l_run += psum;
 
                 bf16x8 pf[4];
 #pragma unroll
@@ -316,15 +297,20 @@ struct Prefill {
                     if (c2 < 2 * nkb) {
 #pragma unroll
                         for (int d = 0; d < D / 32; ++d) {
-                            // row 32d + ln, 16-byte unit (2*c2 + lh) ^ swizzle(row)
-                            bf16x8 a = as_bf16x8(ld16(Vt + d * 32 * BR_BN + v_rd + (v_sw ^ (((2 * c2) ^ (4 * (d & 1))) << 3))));
-                            o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[c2], o[d], 0, 0, 0);
+                            // dims 32d + (lane & 31), keys 16*c2 + 8*lh + 0..3 and + 4..7
+                            const char* vp = stage + L.vrd[d] + c2 * 16 * SM::rowB;
+                            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)vp);
+                            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (lds_s16x4*)(__attribute__((address_space(3))) const char*)(vp + 4 * SM::rowB));
+                            union { s16x8 s8; bf16x8 b8; } a;
+                            a.s8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                            o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b8, pf[c2], o[d], 0, 0, 0);
                         }
                     }
                 }
             }
 
-            if (have_next) store_tile(st, L, smem + (bufi ^ 1) * SM::bufBytes);
+            vm_wait_all();
             __syncthreads();
             bufi ^= 1;
             cur = nxt;
@@ -386,36 +372,36 @@ struct Prefill {
 
 template <int D, int NW>
 __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillParams p) {
-    __shared__ __attribute__((aligned(16))) char smem[Smem<D>::total(NW)];
-    __shared__ int s_ticket;
+    // one LDS object, so that it starts at LDS address 0 and every DMA target stays below 64 KiB;
+    // the ticket mailbox sits behind the tile stages
+    __shared__ __attribute__((aligned(1024))) char smem[Smem<D>::total(NW) + 64];
+    int& s_next = *reinterpret_cast<int*>(smem + Smem<D>::total(NW));
     using PF = Prefill<D, NW>;
+    const int NHG = p.geom.NHG;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
-    const int n_work = pv.hdr[BR_PH_NITEMS] * p.geom.NHG;
-    const typename PF::Lane L = PF::make_lane(p, threadIdx.x);
-    if (threadIdx.x == 0) s_ticket = atomicAdd(&hdr[BR_PH_TICKET], 1);
+    const typename PF::Lane L = PF::make_lane(p, uni(threadIdx.x >> 6), threadIdx.x & 63);
+    // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
+    for (int i = threadIdx.x * 16; i < Smem<D>::total(NW); i += NW * 64 * 16) *reinterpret_cast<uint4*>(smem + i) = uint4{0u, 0u, 0u, 0u};
+    const int xcc = br_xcc_id();
+    int qk = 0;            // step in the queue order (global, this XCD's, the others) thread 0 is at
+    if (threadIdx.x == 0) s_next = br_take_ticket(hdr, NHG, xcc, &qk, -1);
     __syncthreads();
     for (;;) {
-        const int w = uni(s_ticket);
+        const int qt = uni(s_next);
         __syncthreads();
-        if (w >= n_work) break;
-        // the next ticket is fetched now and only looked at after the item: its latency is hidden
-        int next_w = 0;
-        if (threadIdx.x == 0) next_w = atomicAdd(&hdr[BR_PH_TICKET], 1);
-        const int item = w / p.geom.NHG, hg = w - item * p.geom.NHG;
+        if (qt < 0) break;
+        // the next ticket is drawn now and only looked at after the item: its latency is hidden
+        int t_next = -1;
+        if (threadIdx.x == 0 && qk < BR_NQUEUES) t_next = atomicAdd(&hdr[BR_PH_QTICKET + br_queue_at(qk, xcc)], 1);
+        int item, hg;
+        br_decode_ticket(pv, qt, NHG, item, hg);
         const BrItem it = pv.items[item];
         PF::run_item(p, pv, it, hg, smem, L);
-        if (threadIdx.x == 0) s_ticket = next_w;
+        if (threadIdx.x == 0) s_next = br_take_ticket(hdr, NHG, xcc, &qk, t_next);
         __syncthreads();
     }
-    // the last workgroup to leave re-arms the counters for the next launch on this plan
-    if (threadIdx.x == 0) {
-        int d = atomicAdd(&hdr[BR_PH_DONE], 1);
-        if (d == (int)gridDim.x - 1) {
-            atomicExch(&hdr[BR_PH_TICKET], 0);
-            atomicExch(&hdr[BR_PH_DONE], 0);
-        }
-    }
+    if (threadIdx.x == 0) br_leave(hdr);
 }
 
 // Finish: (1) merge the split-KV partials of the query block,

@@ -126,7 +126,7 @@ def test_repeated_calls_reuse_the_plan():
     for o in outs[1:]:
         assert torch.equal(o, outs[0])
     plan = bm.plan(8, 2)
-    assert plan[2].item() == 0 and plan[3].item() == 0     # ticket counters re-armed
+    assert plan[48].item() == 0 and (plan[32:41] == 0).all()     # done and ticket counters re-armed
 
 
 def test_config2_full_size():
