@@ -16,8 +16,10 @@
 #define BR_MIN_CHUNK 4        // a split of the query block's key walk covers at least this many tiles
 
 // Plan buffer (int32):
-//   [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][queue lists 9*max_items]
-//   [items 16*max_items][comb 4*max_comb]
+//   [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
+//   [queue lists 9*max_items][items 16*max_items][comb 4*max_comb]
+// Tile descriptors: for each sequence, the 64-key tiles of blocks 0..M-2 in order, as (token index of
+// the tile's first key, number of real keys); TPS = (M-1) * ceil(H/64) slots per sequence.
 // Work is handed out through 9 queues.  Queue 8 holds the query-block items (the long ones, with no
 // locality preference: they read every key); every workgroup drains it first.  Queues 0..7 belong
 // to the 8 XCDs: all query tiles of one (sequence, block) go to one queue, so the block's K/V for all
@@ -40,13 +42,14 @@ enum BrPlanHeader {
 };
 
 // One unit of prefill work: query tile [t0, t0+T) of block m of sequence b, restricted to a range
-// of its key/value tile walk.  li0/kt0 locate the first tile (walk-list position, tile inside it),
-// ntiles is how many tiles to process (INT_MAX = to the end).  slot < 0: the item owns its rows and
-// writes the final output; slot >= 0: it writes an unnormalised partial into that slot.
-// The item also carries what the kernel would otherwise have to look up in the block table before it
-// can issue its first load: the block's own span and the prefix block's span.
+// of its key/value tile walk.  The walk is: the nprev tiles of the earlier blocks the block may see
+// (the sequence's first nprev tile descriptors), then the tiles of its own block up to the diagonal.
+// f_lo is the first tile of the range in that order, ntiles how many to process (INT_MAX = to the
+// end).  slot < 0: the item owns its rows and writes the final output; slot >= 0: it writes an
+// unnormalised partial into that slot.  The item also carries what the kernel would otherwise have
+// to look up before it can issue its first load: the block's own span and the prefix block's span.
 struct BrItem {
-    int b, m, t0, li0, kt0, ntiles, slot, pe;
+    int b, m, t0, f_lo, nprev, ntiles, slot, pe;
     int len_m, start_m, len0, start0;
     int pad[4];
 };
@@ -59,6 +62,8 @@ struct BrPlanView {
     const int* hdr;
     const int* start;      // B*M
     const int* len;        // B*M
+    const int2* tiles;     // B * TPS tile descriptors
+    int tps;
     const int* qlist;      // 9 lists of item indices, max_items entries apart
     int max_items;
     const BrItem* items;
@@ -74,9 +79,12 @@ __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
     return B * ((M > 1 ? (M - 1) * qt : 0) + last);
 }
 __host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }
-__host__ __device__ inline size_t br_plan_off_qlist(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B; }
+__host__ __device__ inline int br_plan_tps(int M, int H) { return (M > 1 ? M - 1 : 0) * ((H + BR_BN - 1) / BR_BN); }
+__host__ __device__ inline size_t br_plan_off_tbase(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B; }
+__host__ __device__ inline size_t br_plan_off_tiles(int B, int M) { return (br_plan_off_tbase(B, M) + (size_t)B * M + 1) & ~(size_t)1; }
+__host__ __device__ inline size_t br_plan_off_qlist(int B, int M, int H) { return br_plan_off_tiles(B, M) + 2 * (size_t)B * br_plan_tps(M, H); }
 __host__ __device__ inline size_t br_plan_off_items(int B, int M, int H, int T) {
-    size_t o = br_plan_off_qlist(B, M) + (size_t)BR_NQUEUES * br_plan_max_items(B, M, H, T);
+    size_t o = br_plan_off_qlist(B, M, H) + (size_t)BR_NQUEUES * br_plan_max_items(B, M, H, T);
     return (o + 15) & ~(size_t)15;   // 64-byte aligned items
 }
 __host__ __device__ inline size_t br_plan_off_comb(int B, int M, int H, int T) {
@@ -91,7 +99,9 @@ __device__ inline BrPlanView br_plan_view(const int* plan, int B, int M, int H, 
     v.hdr = plan;
     v.start = plan + br_plan_off_start();
     v.len = plan + br_plan_off_len(B, M);
-    v.qlist = plan + br_plan_off_qlist(B, M);
+    v.tiles = reinterpret_cast<const int2*>(plan + br_plan_off_tiles(B, M));
+    v.tps = br_plan_tps(M, H);
+    v.qlist = plan + br_plan_off_qlist(B, M, H);
     v.max_items = br_plan_max_items(B, M, H, T);
     v.items = reinterpret_cast<const BrItem*>(plan + br_plan_off_items(B, M, H, T));
     v.comb = reinterpret_cast<const BrComb*>(plan + br_plan_off_comb(B, M, H, T));
@@ -147,50 +157,52 @@ __host__ __device__ inline int br_prev_blocks(int m, int M) {
     return m == M - 1 ? M - 1 : 1;
 }
 
-// Walk over the key/value tiles one query tile sees: all tiles of blocks 0..pe-1 (full visibility),
-// then the tiles of its own block up to the diagonal.  Every field is uniform across the workgroup.
+// Walk over the key/value tiles one query tile sees.  Every field is uniform across the workgroup.
 struct BrTile {
-    int blk;      // block the tile's keys live in
-    int kt;       // tile index inside that block (valid-relative key kt*BR_BN is its first key)
+    int tok0;     // token index (inside the sequence) of the tile's first key
+    int kt;       // for the block's own tiles: tile index inside the block (first key is kt*BR_BN)
     int nvalid;   // real keys in the tile (1..BR_BN)
     int self;     // 1 if the keys belong to the query tile's own block (causal rule applies)
 };
 
+// Index part of the walk: which tile comes next and whether it is one of the nprev earlier-block
+// tiles (flat index returned in *prev_index, descriptor to be supplied by the caller) or one of the
+// block's own.
 struct BrWalk {
-    const int* len;   // lengths of this sequence's blocks
-    int pe, m, self_end, len0;
-    int li, kt, left;
+    int f, f_end, nprev, self_end, own_tok0;
 
-    __device__ void init(const int* len_b, const BrItem& it, int self_end_) {
-        len = len_b;
-        m = it.m;
-        pe = it.pe;
-        len0 = it.len0;
+    __device__ void init(const BrItem& it, int self_end_, int H) {
+        f = it.f_lo;
+        f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
+        nprev = it.nprev;
         self_end = self_end_;
-        li = it.li0;
-        kt = it.kt0;
-        left = it.ntiles;
+        own_tok0 = it.m * H + it.start_m;
     }
-    __device__ bool next(BrTile& t) {
-        if (left <= 0) return false;
-        while (li <= pe) {
-            int L = li < pe ? (li == 0 ? len0 : len[li]) : self_end;
-            int k0 = kt * BR_BN;
-            if (k0 < L) {
-                t.blk = li < pe ? li : m;
-                t.kt = kt;
-                t.nvalid = L - k0 < BR_BN ? L - k0 : BR_BN;
-                t.self = li == pe;
-                ++kt;
-                --left;
-                return true;
-            }
-            ++li;
-            kt = 0;
+    // returns 0: exhausted, 1: earlier-block tile *prev_index, 2: own tile filled into t
+    __device__ int next(BrTile& t, int* prev_index) {
+        if (f >= f_end) return 0;
+        if (f < nprev) {
+            *prev_index = f++;
+            return 1;
         }
-        return false;
+        const int kt = f - nprev, k0 = kt * BR_BN;
+        if (k0 >= self_end) return 0;
+        t.tok0 = own_tok0 + k0;
+        t.kt = kt;
+        t.nvalid = self_end - k0 < BR_BN ? self_end - k0 : BR_BN;
+        t.self = 1;
+        ++f;
+        return 2;
     }
 };
+
+// Descriptor of earlier-block tile i of a document (the only earlier block is the prefix).
+__device__ inline void br_prefix_tile(const BrItem& it, int i, BrTile& t) {
+    t.tok0 = it.start0 + i * BR_BN;
+    t.kt = i;
+    t.nvalid = it.len0 - i * BR_BN < BR_BN ? it.len0 - i * BR_BN : BR_BN;
+    t.self = 0;
+}
 
 // Row mapping shared by every kernel that touches a work item: a workgroup of NW "row blocks" of 32
 // query rows covers Gw = NW / tpb heads x T = 32 * tpb tokens.  Row block r is head r / tpb of the

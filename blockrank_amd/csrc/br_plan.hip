@@ -82,7 +82,10 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     int* start = plan + br_plan_off_start();
     int* len = plan + br_plan_off_len(B, M);
     int* prev_tiles = plan + br_plan_off_prev(B, M);
-    int* qlist = plan + br_plan_off_qlist(B, M);
+    int* tbase = plan + br_plan_off_tbase(B, M);
+    int2* tiles = reinterpret_cast<int2*>(plan + br_plan_off_tiles(B, M));
+    const int tps = br_plan_tps(M, H);
+    int* qlist = plan + br_plan_off_qlist(B, M, H);
     const int max_items = br_plan_max_items(B, M, H, T);
     BrItem* items = reinterpret_cast<BrItem*>(plan + br_plan_off_items(B, M, H, T));
     BrComb* comb = reinterpret_cast<BrComb*>(plan + br_plan_off_comb(B, M, H, T));
@@ -101,8 +104,20 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     __syncthreads();
     for (int b = tid; b < B; b += kPlanThreads) {
         int s = 0;
-        for (int m = 0; m < M - 1; ++m) s += ceil_div(len[b * M + m], BR_BN);
+        for (int m = 0; m < M - 1; ++m) {
+            tbase[b * M + m] = s;
+            s += ceil_div(len[b * M + m], BR_BN);
+        }
         prev_tiles[b] = s;
+    }
+    __syncthreads();
+    // tile descriptors of blocks 0..M-2, one thread per block
+    for (int p = tid; p < BM; p += kPlanThreads) {
+        const int b = p / M, m = p - b * M;
+        if (m == M - 1) continue;
+        const int L = len[p], st = start[p];
+        for (int kt = 0; kt * BR_BN < L; ++kt)
+            tiles[(size_t)b * tps + tbase[p] + kt] = make_int2(m * H + st + kt * BR_BN, L - kt * BR_BN < BR_BN ? L - kt * BR_BN : BR_BN);
     }
     __syncthreads();
 
@@ -161,13 +176,14 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
             it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
             if (!is_last) {
+                it.nprev = pe > 0 ? ceil_div(it.len0, BR_BN) : 0;
                 for (int tt = 0; tt < nq; ++tt) {
-                    it.t0 = tt * T; it.li0 = 0; it.kt0 = 0;
+                    it.t0 = tt * T; it.f_lo = 0;
                     it.ntiles = 0x7fffffff; it.slot = -1;
                     items[off_i + tt] = it;
                 }
             } else {
-                const int* len_b = len + b * M;
+                it.nprev = pt;
                 int slot = 0;
                 for (int tt = 0; tt < nq; ++tt) {
                     int e = (tt + 1) * T < L ? (tt + 1) * T : L;
@@ -179,19 +195,11 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                         c.b = b; c.t0 = tt * T; c.slot0 = slot; c.nsplit = ns;
                         comb[off_c++] = c;
                     }
-                    // walk-list cursor: position li, tiles before it cum
-                    int li = 0, cum = 0;
                     for (int s = 0; s < ns; ++s) {
                         int lo = (int)((long long)s * nt / ns);
                         int hi = (int)((long long)(s + 1) * nt / ns);
-                        for (;;) {
-                            int tl = li < pe ? ceil_div(len_b[li], BR_BN) : nself;
-                            if (li >= pe || lo < cum + tl) break;
-                            cum += tl;
-                            ++li;
-                        }
-                        it.t0 = tt * T; it.li0 = li; it.kt0 = lo - cum;
-                        it.ntiles = hi - lo; it.slot = ns > 1 ? slot + s : -1;
+                        it.t0 = tt * T; it.f_lo = lo;
+                        it.ntiles = ns > 1 ? hi - lo : 0x7fffffff; it.slot = ns > 1 ? slot + s : -1;
                         items[off_i++] = it;
                     }
                     if (ns > 1) slot += ns;

@@ -43,13 +43,11 @@ __global__ __launch_bounds__(NW * 64) void br_prefill_f32_kernel(BrPrefillParams
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
         const int head = kvh * ge.G + hsub * ge.Gw + g;
-        const int* len_b = pv.len + b * p.M;
-        const int* start_b = pv.start + b * p.M;
-        const int len_m = len_b[m];
+        const int len_m = it.len_m;
         const int row = it.t0 + sub * BR_RB + n;           // this lane pair's query row, valid-relative
         const bool row_ok = row < len_m;
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
-        const int qtok0 = m * p.H + start_b[m];
+        const int qtok0 = m * p.H + it.start_m;
 
         float q[HD], o[HD];
         {
@@ -65,10 +63,22 @@ __global__ __launch_bounds__(NW * 64) void br_prefill_f32_kernel(BrPrefillParams
         const float* vbase = V + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
 
         BrWalk walk;
-        walk.init(len_b, it, self_end);
+        walk.init(it, self_end, p.H);
+        const int2* tiles_b = pv.tiles + (size_t)b * pv.tps;
         BrTile t;
-        while (walk.next(t)) {
-            const int tok0 = t.blk * p.H + start_b[t.blk] + t.kt * BR_BN;
+        for (;;) {
+            int pi = 0;
+            const int wr = walk.next(t, &pi);
+            if (wr == 0) break;
+            if (wr == 1) {
+                if (it.pe > 1) {
+                    const int2 d = tiles_b[pi];
+                    t.tok0 = d.x; t.nvalid = d.y; t.kt = 0; t.self = 0;
+                } else {
+                    br_prefix_tile(it, pi, t);
+                }
+            }
+            const int tok0 = t.tok0;
             __syncthreads();   // previous tile fully consumed
             for (int ch = tid; ch < BR_BN * (D / 4); ch += NT) {
                 int r = ch / (D / 4), c4 = ch - r * (D / 4);

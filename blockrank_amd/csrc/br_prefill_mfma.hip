@@ -89,16 +89,21 @@ struct Prefill {
     using SM = Smem<D>;
 
     // Per-lane constants, fixed for the whole kernel.
+    // With 4 or 8 waves the DMA pieces of one lane are a whole number of 16-row groups apart, so one
+    // offset plus a uniform step describes them all; otherwise each piece keeps its own offset.
+    static constexpr bool UNIFORM_STEP = (NW == 4 || NW == 8);
+    static constexpr int JO = UNIFORM_STEP ? 1 : JK;
+    static constexpr int STEP_ROWS = NW * 64 / CPR;        // rows between consecutive pieces of a wave
     struct Lane {
-        int koff[JK], voff[JK];    // global byte offsets inside a tile of this lane's DMA pieces
-        int krd[D / 16];           // LDS byte offsets of the K operand reads, one per 16-dim chunk
+        int koff[JO], voff[JO];    // global byte offsets inside a tile of this lane's DMA pieces
+        int krd;                   // LDS byte offset of the K operand read of chunk 0; chunk c is krd ^ (c << 5)
         int vrd[D / 32];           // LDS byte offsets of the V^T operand reads, one per 32-dim block
     };
 
     static __device__ inline Lane make_lane(const BrPrefillParams& p, int wave, int lane) {
         Lane L;
 #pragma unroll
-        for (int j = 0; j < JK; ++j) {
+        for (int j = 0; j < JO; ++j) {
             const int slot = (wave + NW * j) * 64 + lane;
             const int prow = slot / CPR, cp = slot - prow * CPR;
             const int kkey = (prow & 32) | swap23(prow & 31);
@@ -106,8 +111,7 @@ struct Prefill {
             L.voff[j] = prow * (int)p.sv_t * 2 + ((cp ^ ((prow & 3) << 1)) << 4);
         }
         const int ln = lane & 31, lh = lane >> 5;
-#pragma unroll
-        for (int c = 0; c < D / 16; ++c) L.krd[c] = ln * SM::rowB + (((2 * c + lh) ^ (ln & 7)) << 4);
+        L.krd = ln * SM::rowB + ((lh ^ (ln & 7)) << 4);
         // transposing read: within a group of 16 lanes, lane s points at key (s >> 2), dims 4 * (s & 3)
         const int s = lane & 15, ln_hi = (lane >> 4) & 1;
         const int cl = (2 * ln_hi + ((s & 3) >> 1)) ^ ((s >> 2) << 1);
@@ -125,8 +129,13 @@ struct Prefill {
             for (int j = 0; j < JK; ++j) {
                 const int q = wave + NW * j;
                 if (NI % NW == 0 || q < NI) {
-                    dma16(kt, L.koff[j], stage_lds + q * 1024);
-                    dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
+                    if (UNIFORM_STEP) {
+                        dma16(reinterpret_cast<const char*>(kt) + j * STEP_ROWS * sk_bytes, L.koff[0], stage_lds + q * 1024);
+                        dma16(reinterpret_cast<const char*>(vt) + j * STEP_ROWS * sv_bytes, L.voff[0], stage_lds + SM::kBytes + q * 1024);
+                    } else {
+                        dma16(kt, L.koff[j], stage_lds + q * 1024);
+                        dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
+                    }
                 }
             }
         } else {
@@ -136,8 +145,118 @@ struct Prefill {
             for (int j = 0; j < JK; ++j) {
                 const int q = wave + NW * j;
                 if (NI % NW == 0 || q < NI) {
-                    if (L.koff[j] < nvalid * sk_bytes) dma16(kt, L.koff[j], stage_lds + q * 1024);
-                    if (L.voff[j] < nvalid * sv_bytes) dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
+                    const int ko = UNIFORM_STEP ? L.koff[0] + j * STEP_ROWS * sk_bytes : L.koff[j];
+                    const int vo = UNIFORM_STEP ? L.voff[0] + j * STEP_ROWS * sv_bytes : L.voff[j];
+                    if (ko < nvalid * sk_bytes) dma16(kt, ko, stage_lds + q * 1024);
+                    if (vo < nvalid * sv_bytes) dma16(vt, vo, stage_lds + SM::kBytes + q * 1024);
+                }
+            }
+        }
+    }
+
+    static __device__ inline bf16x8 read_k(const char* stage, const Lane& L, int kb, int c) {
+        return as_bf16x8(ld16(stage + kb * 32 * SM::rowB + (L.krd ^ (c << 5))));
+    }
+    // V^T operand for dims 32d + (lane & 31), keys 16*c2 + 8*lh + 0..7: two transposing reads
+    static __device__ inline bf16x8 read_vt(const char* stage, const Lane& L, int d, int c2) {
+        const char* vp = stage + L.vrd[d] + c2 * 16 * SM::rowB;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)vp);
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)(vp + 4 * SM::rowB));
+        union { s16x8 s8; bf16x8 b8; } a;
+        a.s8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return a.b8;
+    }
+
+    // One wave, one 64-key tile already in LDS: S^T = K Q^T, online softmax, O^T += V^T P^T.
+    // FULL: all 64 keys are visible to every row (the common case), one straight-line block with the
+    // LDS operand reads issued several MFMAs ahead of their use.  Otherwise nkb 32-key halves are
+    // computed and keys >= lim are masked per row.
+    template <bool FULL>
+    static __device__ inline void compute_tile(const char* stage, const Lane& L, const bf16x8 (&qf)[D / 16], f32x16 (&o)[D / 32],
+                                               float& m_run, float& l_run, float scale_log2, int nkb, int lim, int lh) {
+        constexpr int NC = D / 16, ND = D / 32;
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        f32x16 s[2];
+        if (FULL) {
+            // the two key halves alternate so that consecutive MFMAs are independent; reads run 4 ahead
+            bf16x8 ka[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ka[i] = read_k(stage, L, i & 1, i >> 1);
+            s[0] = zero;
+            s[1] = zero;
+#pragma unroll
+            for (int i = 0; i < 2 * NC; ++i) {
+                const bf16x8 a = ka[i & 3];
+                if (i + 4 < 2 * NC) ka[i & 3] = read_k(stage, L, (i + 4) & 1, (i + 4) >> 1);
+                s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[i >> 1], s[i & 1], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if (kb < nkb) {
+                    f32x16 acc = zero;
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_k(stage, L, kb, c), qf[c], acc, 0, 0, 0);
+                    s[kb] = acc;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[kb][v] = -INFINITY;
+                }
+            }
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int key = kb * 32 + 16 * (v >> 3) + 8 * lh + (v & 7);
+                    if (key >= lim) s[kb][v] = -INFINITY;
+                }
+        }
+        // first V^T operands: their LDS latency passes under the softmax arithmetic
+        bf16x8 va[ND];
+#pragma unroll
+        for (int d = 0; d < ND; ++d) va[d] = read_vt(stage, L, d, 0);
+
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        // Lazy rescale: the running max is only raised (and O, l rescaled) when some row's max grew by
+        // more than 2^8; otherwise exponentials are taken against the older max, which changes nothing
+        // in the final quotient and keeps them below 2^8.
+        const float m_new = fmaxf(m_run, mx * scale_log2);
+        if (__builtin_amdgcn_ballot_w64(m_new - m_run > 8.f) != 0) {
+            const float m_sub = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_sub);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int d = 0; d < ND; ++d)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
+        }
+        const float m_sub = m_run == -INFINITY ? 0.f : m_run;
+        float psum = 0.f;
+        bf16x8 pf[4];
+#pragma unroll
+        for (int c2 = 0; c2 < 4; ++c2) {
+            f32x8 t;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                t[e] = __builtin_amdgcn_exp2f(s[c2 >> 1][8 * (c2 & 1) + e] * scale_log2 - m_sub);
+                psum += t[e];
+            }
+            pf[c2] = __builtin_convertvector(t, bf16x8);
+        }
+        l_run += psum;
+#pragma unroll
+        for (int c2 = 0; c2 < 4; ++c2) {
+            if (FULL || c2 < 2 * nkb) {
+#pragma unroll
+                for (int d = 0; d < ND; ++d) {
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d], pf[c2], o[d], 0, 0, 0);
+                    if (c2 + 1 < 4 && (FULL || c2 + 1 < 2 * nkb)) va[d] = read_vt(stage, L, d, c2 + 1);
                 }
             }
         }
@@ -153,8 +272,6 @@ struct Prefill {
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
         const int head = kvh * ge.G + hsub * ge.Gw + g;
-        const int* len_b = pv.len + b * p.M;
-        const int* start_b = pv.start + b * p.M;
         const int len_m = it.len_m;
         const int row0 = it.t0 + sub * BR_RB;              // first query row of this wave, valid-relative
         const bool rb_active = row0 < len_m;
@@ -166,14 +283,41 @@ struct Prefill {
         const __bf16* kbase = reinterpret_cast<const __bf16*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h;
         const __bf16* vbase = reinterpret_cast<const __bf16*>(p.v) + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
 
+        // The walk needs no memory lookups inside the loop: a document's only earlier block is the
+        // prefix (described by the item itself); a query-block item keeps the descriptors of its
+        // earlier-block tiles in lane registers (lane i = tile dbase + i) and reads them with readlane.
         BrWalk walk;
-        walk.init(len_b, it, self_end);
+        walk.init(it, self_end, p.H);
+        const int2* tiles_b = pv.tiles + (size_t)b * pv.tps;
+        const bool table = it.pe > 1;
+        int dbase = it.f_lo;
+        int2 dreg = make_int2(0, 0);
+        if (table && dbase + lane < it.nprev) dreg = tiles_b[dbase + lane];
+        auto fetch = [&](BrTile& t) -> bool {
+            int pi = 0;
+            const int r = walk.next(t, &pi);
+            if (r == 0) return false;
+            if (r == 1) {
+                if (!table) {
+                    br_prefix_tile(it, pi, t);
+                } else {
+                    if (pi - dbase >= 64) {
+                        dbase = pi;
+                        dreg = dbase + lane < it.nprev ? tiles_b[dbase + lane] : make_int2(0, 0);
+                        asm volatile("" : "+v"(dreg.x), "+v"(dreg.y));   // wait here, not at every later use
+                    }
+                    t.tok0 = __builtin_amdgcn_readlane(dreg.x, pi - dbase);
+                    t.nvalid = __builtin_amdgcn_readlane(dreg.y, pi - dbase);
+                    t.kt = 0;
+                    t.self = 0;
+                }
+            }
+            return true;
+        };
         BrTile cur, nxt;
-        bool have = walk.next(cur);
-        if (have) {
-            const long long tok0 = cur.blk * p.H + (cur.blk == m ? it.start_m : (cur.blk == 0 ? it.start0 : start_b[cur.blk])) + cur.kt * BR_BN;
-            issue_tile(L, wave, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, sk_bytes, sv_bytes, cur.nvalid, smem_lds);
-        }
+        bool have = fetch(cur);
+        if (have)
+            issue_tile(L, wave, kbase + (long long)cur.tok0 * p.sk_t, vbase + (long long)cur.tok0 * p.sv_t, sk_bytes, sv_bytes, cur.nvalid, smem_lds);
 
         // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.
         bf16x8 qf[D / 16];
@@ -198,16 +342,19 @@ struct Prefill {
         float m_run = -INFINITY, l_run = 0.f;
 
         vm_wait_all();
+        // tell the compiler the Q fragments are in registers now: otherwise it would put its own
+        // "wait for every outstanding load" in front of the first MFMA of each iteration, which would
+        // also wait for the next tile's DMA and undo the overlap
+#pragma unroll
+        for (int c = 0; c < D / 16; ++c) asm volatile("" : "+v"(qf[c]));
         __syncthreads();
         int bufi = 0;
 
         while (have) {
-            const bool have_next = walk.next(nxt);
-            if (have_next) {
-                const long long tok0 = nxt.blk * p.H + (nxt.blk == m ? it.start_m : (nxt.blk == 0 ? it.start0 : start_b[nxt.blk])) + nxt.kt * BR_BN;
-                issue_tile(L, wave, kbase + tok0 * p.sk_t, vbase + tok0 * p.sv_t, sk_bytes, sv_bytes, nxt.nvalid,
-                           smem_lds + (bufi ^ 1) * SM::stageBytes);
-            }
+            const bool have_next = fetch(nxt);
+            if (have_next)
+                issue_tile(L, wave, kbase + (long long)nxt.tok0 * p.sk_t, vbase + (long long)nxt.tok0 * p.sv_t, sk_bytes, sv_bytes,
+                           nxt.nvalid, smem_lds + (bufi ^ 1) * SM::stageBytes);
             const char* stage = smem + bufi * SM::stageBytes;
 
             // 32-key halves of the tile this wave needs: limited by the real keys in the tile and, on
@@ -220,94 +367,13 @@ struct Prefill {
                 nkb = c < nkb ? c : nkb;
             }
             if (!rb_active) nkb = 0;
-
-            if (nkb > 0) {
-                f32x16 s[2];
-                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    if (kb < nkb) {
-                        f32x16 acc = zero;
-#pragma unroll
-                        for (int c = 0; c < D / 16; ++c) {
-                            bf16x8 a = as_bf16x8(ld16(stage + kb * 32 * SM::rowB + L.krd[c]));
-                            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], acc, 0, 0, 0);
-                        }
-                        s[kb] = acc;
-                    } else {
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) s[kb][v] = -INFINITY;
-                    }
-                }
-                // mask keys past the tile's real keys and beyond the diagonal
-                const bool need_mask = (cur.nvalid < nkb * 32) || (cur.self && key0 + nkb * 32 - 1 > row0);
-                if (need_mask) {
-                    const int lim_causal = cur.self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
-                    const int lim = cur.nvalid < lim_causal ? cur.nvalid : lim_causal;
-#pragma unroll
-                    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            int key = kb * 32 + 16 * (v >> 3) + 8 * lh + (v & 7);
-                            if (key >= lim) s[kb][v] = -INFINITY;
-                        }
-                }
-                float mx = -INFINITY;
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32));
-                // Lazy rescale: the running max is only raised (and O, l rescaled) when some row's max
-                // grew by more than 2^8; otherwise exponentials are taken against the older max, which
-                // changes nothing in the final quotient and keeps them below 2^8.
-                const float m_new = fmaxf(m_run, mx * p.scale_log2);
-                if (__builtin_amdgcn_ballot_w64(m_new - m_run > 8.f) != 0) {
-                    const float m_sub = m_new == -INFINITY ? 0.f : m_new;
-                    const float alpha = __builtin_amdgcn_exp2f(m_run - m_sub);
-                    m_run = m_new;
-                    l_run *= alpha;
-#pragma unroll
-                    for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
-                }
-                const float m_sub = m_run == -INFINITY ? 0.f : m_run;
-                float psum = 0.f;
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        float e = __builtin_amdgcn_exp2f(s[kb][v] * p.scale_log2 - m_sub);
-                        s[kb][v] = e;
-                        psum += e;
-                    }
-                l_run += psum;
-
-                bf16x8 pf[4];
-#pragma unroll
-                for (int c2 = 0; c2 < 4; ++c2) {
-                    f32x8 t;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) t[e] = s[c2 >> 1][8 * (c2 & 1) + e];
-                    pf[c2] = __builtin_convertvector(t, bf16x8);
-                }
-#pragma unroll
-                for (int c2 = 0; c2 < 4; ++c2) {
-                    if (c2 < 2 * nkb) {
-#pragma unroll
-                        for (int d = 0; d < D / 32; ++d) {
-                            // dims 32d + (lane & 31), keys 16*c2 + 8*lh + 0..3 and + 4..7
-                            const char* vp = stage + L.vrd[d] + c2 * 16 * SM::rowB;
-                            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)vp);
-                            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                (lds_s16x4*)(__attribute__((address_space(3))) const char*)(vp + 4 * SM::rowB));
-                            union { s16x8 s8; bf16x8 b8; } a;
-                            a.s8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                            o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b8, pf[c2], o[d], 0, 0, 0);
-                        }
-                    }
-                }
+            const bool need_mask = (cur.nvalid < nkb * 32) || (cur.self && key0 + nkb * 32 - 1 > row0);
+            if (nkb == 2 && !need_mask) {
+                compute_tile<true>(stage, L, qf, o, m_run, l_run, p.scale_log2, 2, 0, lh);
+            } else if (nkb > 0) {
+                const int lim_causal = cur.self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
+                const int lim = need_mask ? (cur.nvalid < lim_causal ? cur.nvalid : lim_causal) : BR_BN;
+                compute_tile<false>(stage, L, qf, o, m_run, l_run, p.scale_log2, nkb, lim, lh);
             }
 
             vm_wait_all();
