@@ -48,6 +48,9 @@ def workloads():
         # BASELINE configs[4] shapes with bf16 QK^T (the fp8 variant is not built)
         "cfg5shape": dict(desc="Qwen2.5-7B attention shapes, B=4, 28q/4kv heads, D=128, 32-token prefix + 50 lognormal docs + 24-token query, bf16",
                           layout=lambda: synthetic.lognormal_layout(4, 32, 50, 120, 0.6, 16, 512, 24, seed=0), Nq=28, Nkv=4, D=128, hidden=3584, dtype=torch.bfloat16),
+        # one long causal block per sequence: many key tiles per work item (steady-state tile throughput)
+        "causal4k": dict(desc="single block of 4096 tokens per sequence (plain causal), B=8, 32q/8kv heads, D=128, bf16",
+                         layout=lambda: synthetic.make_layout([[4096]] * 8), Nq=32, Nkv=8, D=128, hidden=None, dtype=torch.bfloat16),
         # BASELINE configs[0]: the reference's CPU-runnable case
         "cfg1": dict(desc="fp32, B=1, 8q/2kv heads, D=64, 32-token prefix + 8 docs x 64 + 16-token query", layout=lambda: synthetic.uniform_layout(1, 32, 8, 64, 16),
                      Nq=8, Nkv=2, D=64, hidden=None, dtype=torch.float32),
@@ -133,7 +136,7 @@ def main():
 
     def step(events=None):
         out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events)
-        scores = handle.doc_scores(rows, temperature=0.05)
+        scores = handle.doc_scores(rows, temperature=0.05) if handle is not None else None
         return out, scores
 
     for _ in range(args.warmup):

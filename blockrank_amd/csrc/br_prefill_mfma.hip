@@ -81,6 +81,89 @@ __device__ inline unsigned lds_addr_of(const void* p) {
 // the P^T V product.
 __device__ inline int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
+// Descriptor prefetch, run by wave 0 while the workgroup computes an item: the ticket for the next
+// item is drawn at the start of the current one; after the first key tile the queue list entry is
+// requested, after the second the 64-byte item itself, and at the end of the item it is published
+// through LDS.  Each step consumes a value whose load was issued a whole tile earlier, so the chain
+// ticket -> list entry -> item costs the item's critical path nothing (items with fewer tiles finish
+// the chain at the end, waiting as needed).
+struct BrDescMail {      // layout of one LDS mailbox
+    int word[BR_ITEM_INTS];
+    int hg;
+    int valid;
+    int pad[2];
+};
+
+struct BrPrefetch {
+    int* hdr;
+    const BrPlanView* pv;
+    int NHG, xcc, lane;
+    int qk;        // step in the queue order (global, this XCD's, the others)
+    int counts;    // lane j: work units in queue j
+    int t_next;    // ticket drawn from the queue at step qk (lane 0), or -1
+    int stage;     // 0 ticket drawn, 1 list entry requested, 2 item requested, 9 queue ran dry
+    int idx_v, word, hg;
+
+    __device__ void init(int* hdr_, const BrPlanView* pv_, int NHG_, int lane_) {
+        hdr = hdr_; pv = pv_; NHG = NHG_; lane = lane_;
+        xcc = br_xcc_id();
+        qk = 0;
+        counts = lane < BR_NQUEUES ? hdr[BR_PH_QCOUNT + lane] * NHG : 0;
+        t_next = -1;
+        stage = 9;
+        idx_v = word = hg = 0;
+    }
+    __device__ void draw() {   // at the start of an item
+        t_next = -1;
+        stage = 9;
+        if (qk < BR_NQUEUES) {
+            if (lane == 0) t_next = atomicAdd(&hdr[BR_PH_QTICKET + br_queue_at(qk, xcc)], 1);
+            stage = 0;
+        }
+    }
+    __device__ void step() {   // once per key tile, after the tile's arithmetic
+        if (stage == 0) {
+            const int q = br_queue_at(qk, xcc);
+            const int t = __builtin_amdgcn_readfirstlane(t_next);
+            if (t < __builtin_amdgcn_readlane(counts, q)) {
+                const int li = t / NHG;
+                hg = t - li * NHG;
+                idx_v = pv->qlist[(size_t)q * pv->max_items + li];
+                stage = 1;
+            } else {
+                stage = 9;
+            }
+        } else if (stage == 1) {
+            const int idx = __builtin_amdgcn_readfirstlane(idx_v);
+            word = reinterpret_cast<const int*>(pv->items + idx)[lane & (BR_ITEM_INTS - 1)];
+            stage = 2;
+        }
+    }
+    __device__ void publish(BrDescMail* mail) {   // at the end of an item
+        if (stage == 0) step();
+        if (stage == 1) step();
+        if (stage == 9) {
+            // the queue ran dry (or nothing was drawn): look through the remaining queues now
+            int qt = -1;
+            if (lane == 0) qt = br_take_ticket(hdr, NHG, xcc, &qk, t_next);
+            qt = __builtin_amdgcn_readfirstlane(qt);
+            qk = __builtin_amdgcn_readfirstlane(qk);
+            if (qt < 0) {
+                if (lane == 0) mail->valid = 0;
+                return;
+            }
+            int item;
+            br_decode_ticket(*pv, qt, NHG, item, hg);
+            word = reinterpret_cast<const int*>(pv->items + item)[lane & (BR_ITEM_INTS - 1)];
+        }
+        if (lane < BR_ITEM_INTS) mail->word[lane] = word;
+        if (lane == 0) {
+            mail->hg = hg;
+            mail->valid = 1;
+        }
+    }
+};
+
 template <int D, int NW>
 struct Prefill {
     static constexpr int CPR = D / 8;                      // 16-byte chunks per K/V row
@@ -263,7 +346,7 @@ struct Prefill {
     }
 
     static __device__ void run_item(const BrPrefillParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem,
-                                    const Lane& L) {
+                                    const Lane& L, BrPrefetch& pf) {
         const int tid = threadIdx.x;
         const int wave = uni(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
         const BrGeom& ge = p.geom;
@@ -376,6 +459,7 @@ struct Prefill {
                 compute_tile<false>(stage, L, qf, o, m_run, l_run, p.scale_log2, nkb, lim, lh);
             }
 
+            if (wave == 0) pf.step();
             vm_wait_all();
             __syncthreads();
             bufi ^= 1;
@@ -439,32 +523,33 @@ struct Prefill {
 template <int D, int NW>
 __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillParams p) {
     // one LDS object, so that it starts at LDS address 0 and every DMA target stays below 64 KiB;
-    // the ticket mailbox sits behind the tile stages
-    __shared__ __attribute__((aligned(1024))) char smem[Smem<D>::total(NW) + 64];
-    int& s_next = *reinterpret_cast<int*>(smem + Smem<D>::total(NW));
+    // the two descriptor mailboxes sit behind the tile stages
+    __shared__ __attribute__((aligned(1024))) char smem[Smem<D>::total(NW) + 2 * sizeof(BrDescMail)];
+    BrDescMail* mail = reinterpret_cast<BrDescMail*>(smem + Smem<D>::total(NW));
     using PF = Prefill<D, NW>;
     const int NHG = p.geom.NHG;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
-    const typename PF::Lane L = PF::make_lane(p, uni(threadIdx.x >> 6), threadIdx.x & 63);
+    const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const typename PF::Lane L = PF::make_lane(p, wave, lane);
     // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
     for (int i = threadIdx.x * 16; i < Smem<D>::total(NW); i += NW * 64 * 16) *reinterpret_cast<uint4*>(smem + i) = uint4{0u, 0u, 0u, 0u};
-    const int xcc = br_xcc_id();
-    int qk = 0;            // step in the queue order (global, this XCD's, the others) thread 0 is at
-    if (threadIdx.x == 0) s_next = br_take_ticket(hdr, NHG, xcc, &qk, -1);
+    BrPrefetch pf;
+    pf.init(hdr, &pv, NHG, lane);
+    if (wave == 0) pf.publish(&mail[0]);
     __syncthreads();
-    for (;;) {
-        const int qt = uni(s_next);
-        __syncthreads();
-        if (qt < 0) break;
-        // the next ticket is drawn now and only looked at after the item: its latency is hidden
-        int t_next = -1;
-        if (threadIdx.x == 0 && qk < BR_NQUEUES) t_next = atomicAdd(&hdr[BR_PH_QTICKET + br_queue_at(qk, xcc)], 1);
-        int item, hg;
-        br_decode_ticket(pv, qt, NHG, item, hg);
-        const BrItem it = pv.items[item];
-        PF::run_item(p, pv, it, hg, smem, L);
-        if (threadIdx.x == 0) s_next = br_take_ticket(hdr, NHG, xcc, &qk, t_next);
+    for (int cur = 0;; cur ^= 1) {
+        if (uni(mail[cur].valid) == 0) break;
+        BrItem it;
+        {
+            int* w = reinterpret_cast<int*>(&it);
+#pragma unroll
+            for (int i = 0; i < 12; ++i) w[i] = uni(mail[cur].word[i]);
+        }
+        const int hg = uni(mail[cur].hg);
+        if (wave == 0) pf.draw();
+        PF::run_item(p, pv, it, hg, smem, L, pf);
+        if (wave == 0) pf.publish(&mail[cur ^ 1]);
         __syncthreads();
     }
     if (threadIdx.x == 0) br_leave(hdr);
