@@ -48,6 +48,8 @@ def workloads():
         # BASELINE configs[4] shapes with bf16 QK^T (the fp8 variant is not built)
         "cfg5shape": dict(desc="Qwen2.5-7B attention shapes, B=4, 28q/4kv heads, D=128, 32-token prefix + 50 lognormal docs + 24-token query, bf16",
                           layout=lambda: synthetic.lognormal_layout(4, 32, 50, 120, 0.6, 16, 512, 24, seed=0), Nq=28, Nkv=4, D=128, hidden=3584, dtype=torch.bfloat16),
+        "cfg2_b1": dict(desc="cfg2 with B=1", layout=lambda: synthetic.uniform_layout(1, 64, 20, 160, 32), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
+        "cfg2_b16": dict(desc="cfg2 with B=16", layout=lambda: synthetic.uniform_layout(16, 64, 20, 160, 32), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
         # one long causal block per sequence: many key tiles per work item (steady-state tile throughput)
         "causal4k": dict(desc="single block of 4096 tokens per sequence (plain causal), B=8, 32q/8kv heads, D=128, bf16",
                          layout=lambda: synthetic.make_layout([[4096]] * 8), Nq=32, Nkv=8, D=128, hidden=None, dtype=torch.bfloat16),

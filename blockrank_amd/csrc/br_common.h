@@ -17,14 +17,15 @@
 
 // Plan buffer (int32):
 //   [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
-//   [queue lists 9*max_items][items 16*max_items][comb 4*max_comb]
+//   [items 16*max_items][comb 4*max_comb]
 // Tile descriptors: for each sequence, the 64-key tiles of blocks 0..M-2 in order, as (token index of
 // the tile's first key, number of real keys); TPS = (M-1) * ceil(H/64) slots per sequence.
 // Work is handed out through 9 queues.  Queue 8 holds the query-block items (the long ones, with no
 // locality preference: they read every key); every workgroup drains it first.  Queues 0..7 belong
 // to the 8 XCDs: all query tiles of one (sequence, block) go to one queue, so the block's K/V for all
-// heads are fetched into one XCD's L2 only.  A ticket t of a queue is (list entry t / NHG, head group
-// t % NHG): consecutive tickets cover all kv heads, which keeps every L2 channel busy.
+// heads are fetched into one XCD's L2 only.  The items array is grouped by queue (queue g's items
+// start at QOFF[g]); a ticket t of queue g is (item QOFF[g] + t / NHG, head group t % NHG):
+// consecutive tickets cover all kv heads, which keeps every L2 channel busy.
 #define BR_PLAN_HDR 64
 #define BR_NQUEUES 9
 #define BR_GLOBAL_QUEUE 8
@@ -36,6 +37,7 @@ enum BrPlanHeader {
     BR_PH_MAX_COMB = 6,
     BR_PH_T = 7,          // tokens per query tile the plan was built for
     BR_PH_QCOUNT = 8,     // [9] items in each queue
+    BR_PH_QOFF = 17,      // [9] index of each queue's first item
     // second cache line: everything the running kernels update
     BR_PH_QTICKET = 32,   // [9] ticket counters (zero between launches)
     BR_PH_DONE = 48,      // workgroups that have left the persistent loop (zero between launches)
@@ -64,8 +66,6 @@ struct BrPlanView {
     const int* len;        // B*M
     const int2* tiles;     // B * TPS tile descriptors
     int tps;
-    const int* qlist;      // 9 lists of item indices, max_items entries apart
-    int max_items;
     const BrItem* items;
     const BrComb* comb;
 };
@@ -82,9 +82,8 @@ __host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PE
 __host__ __device__ inline int br_plan_tps(int M, int H) { return (M > 1 ? M - 1 : 0) * ((H + BR_BN - 1) / BR_BN); }
 __host__ __device__ inline size_t br_plan_off_tbase(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B; }
 __host__ __device__ inline size_t br_plan_off_tiles(int B, int M) { return (br_plan_off_tbase(B, M) + (size_t)B * M + 1) & ~(size_t)1; }
-__host__ __device__ inline size_t br_plan_off_qlist(int B, int M, int H) { return br_plan_off_tiles(B, M) + 2 * (size_t)B * br_plan_tps(M, H); }
 __host__ __device__ inline size_t br_plan_off_items(int B, int M, int H, int T) {
-    size_t o = br_plan_off_qlist(B, M, H) + (size_t)BR_NQUEUES * br_plan_max_items(B, M, H, T);
+    size_t o = br_plan_off_tiles(B, M) + 2 * (size_t)B * br_plan_tps(M, H);
     return (o + 15) & ~(size_t)15;   // 64-byte aligned items
 }
 __host__ __device__ inline size_t br_plan_off_comb(int B, int M, int H, int T) {
@@ -101,8 +100,6 @@ __device__ inline BrPlanView br_plan_view(const int* plan, int B, int M, int H, 
     v.len = plan + br_plan_off_len(B, M);
     v.tiles = reinterpret_cast<const int2*>(plan + br_plan_off_tiles(B, M));
     v.tps = br_plan_tps(M, H);
-    v.qlist = plan + br_plan_off_qlist(B, M, H);
-    v.max_items = br_plan_max_items(B, M, H, T);
     v.items = reinterpret_cast<const BrItem*>(plan + br_plan_off_items(B, M, H, T));
     v.comb = reinterpret_cast<const BrComb*>(plan + br_plan_off_comb(B, M, H, T));
     return v;
@@ -138,7 +135,7 @@ __device__ inline void br_decode_ticket(const BrPlanView& pv, int qt, int NHG, i
     const int q = qt >> 24, t = qt & 0xffffff;
     const int li = t / NHG;
     hg = t - li * NHG;
-    item = pv.qlist[(size_t)q * pv.max_items + li];
+    item = pv.hdr[BR_PH_QOFF + q] + li;
 }
 
 // Leave the persistent loop: the last workgroup re-arms the counters for the next launch.

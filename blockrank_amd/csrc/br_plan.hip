@@ -85,7 +85,6 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     int* tbase = plan + br_plan_off_tbase(B, M);
     int2* tiles = reinterpret_cast<int2*>(plan + br_plan_off_tiles(B, M));
     const int tps = br_plan_tps(M, H);
-    int* qlist = plan + br_plan_off_qlist(B, M, H);
     const int max_items = br_plan_max_items(B, M, H, T);
     BrItem* items = reinterpret_cast<BrItem*>(plan + br_plan_off_items(B, M, H, T));
     BrComb* comb = reinterpret_cast<BrComb*>(plan + br_plan_off_comb(B, M, H, T));
@@ -121,7 +120,53 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     }
     __syncthreads();
 
-    // Pairs (sequence, block) are visited sequence by sequence, the query block first.
+    // Pass 1: how many items each queue gets, so that the items array can be laid out queue by queue.
+    int qoff[BR_NQUEUES];
+    {
+        int qtot[BR_NQUEUES];
+#pragma unroll
+        for (int g = 0; g < BR_NQUEUES; ++g) qtot[g] = 0;
+        for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
+            const int p = p0 + tid;
+            int n_items = 0, myq = -1;
+            if (p < BM) {
+                const int b = p / M, jj = p - b * M;
+                const int m = jj == 0 ? M - 1 : jj - 1;
+                const int L = len[b * M + m];
+                const int nq = ceil_div(L, T);
+                if (jj == 0) {
+                    myq = BR_GLOBAL_QUEUE;
+                    const int pt = M > 1 ? prev_tiles[b] : 0;
+                    int ns_cap = nq > 0 ? BR_SLOTS_PER_SEQ / nq : 1;
+                    ns_cap = ns_cap < 1 ? 1 : ns_cap;
+                    for (int tt = 0; tt < nq; ++tt) {
+                        int e = (tt + 1) * T < L ? (tt + 1) * T : L;
+                        n_items += splits_for(pt + ceil_div(e, BR_BN), ns_cap);
+                    }
+                } else {
+                    myq = (b * (M - 1) + m) & 7;
+                    n_items = nq;
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < BR_NQUEUES; ++g) {
+                int tot_g;
+                block_exclusive_scan(myq == g ? n_items : 0, sh, &tot_g);
+                qtot[g] += tot_g;
+            }
+        }
+        // the global queue first, then the XCD queues
+        int c = 0;
+        qoff[BR_GLOBAL_QUEUE] = c;
+        c += qtot[BR_GLOBAL_QUEUE];
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            qoff[g] = c;
+            c += qtot[g];
+        }
+    }
+
+    // Pass 2: pairs (sequence, block) are visited sequence by sequence, the query block first.
     int base_items = 0, base_comb = 0;
     int qbase[BR_NQUEUES];
 #pragma unroll
@@ -155,7 +200,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             }
         }
         int tot_i, tot_c;
-        int off_i = base_items + block_exclusive_scan(n_items, sh, &tot_i);
+        block_exclusive_scan(n_items, sh, &tot_i);
         int off_c = base_comb + block_exclusive_scan(n_comb, sh, &tot_c);
         base_items += tot_i;
         base_comb += tot_c;
@@ -165,11 +210,11 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         for (int g = 0; g < BR_NQUEUES; ++g) {
             int tot_g;
             int r = block_exclusive_scan(myq == g ? n_items : 0, sh, &tot_g);
-            if (myq == g) qpos = qbase[g] + r;
+            if (myq == g) qpos = qoff[g] + qbase[g] + r;
             qbase[g] += tot_g;
         }
         if (p < BM) {
-            for (int k = 0; k < n_items; ++k) qlist[(size_t)myq * max_items + qpos + k] = off_i + k;
+            int off_i = qpos;     // this pair's items sit together inside its queue's run
             const int pe = br_prev_blocks(m, M);
             BrItem it;
             it.b = b; it.m = m; it.pe = pe;
@@ -210,7 +255,10 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     __syncthreads();
     if (tid == 0) {
 #pragma unroll
-        for (int g = 0; g < BR_NQUEUES; ++g) hdr[BR_PH_QCOUNT + g] = qbase[g];
+        for (int g = 0; g < BR_NQUEUES; ++g) {
+            hdr[BR_PH_QCOUNT + g] = qbase[g];
+            hdr[BR_PH_QOFF + g] = qoff[g];
+        }
         hdr[BR_PH_NITEMS] = base_items;
         hdr[BR_PH_NCOMB] = base_comb;
         hdr[BR_PH_NONCONTIG] = s_bad;

@@ -82,11 +82,10 @@ __device__ inline unsigned lds_addr_of(const void* p) {
 __device__ inline int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
 // Descriptor prefetch, run by wave 0 while the workgroup computes an item: the ticket for the next
-// item is drawn at the start of the current one; after the first key tile the queue list entry is
-// requested, after the second the 64-byte item itself, and at the end of the item it is published
-// through LDS.  Each step consumes a value whose load was issued a whole tile earlier, so the chain
-// ticket -> list entry -> item costs the item's critical path nothing (items with fewer tiles finish
-// the chain at the end, waiting as needed).
+// item is drawn at the start of the current one; after the first key tile the 64-byte item it names
+// is requested, and at the end of the item it is published through LDS.  Each step consumes a value
+// whose load was issued a whole tile earlier, so the chain ticket -> item costs the item's critical
+// path nothing (an item with a single tile finishes the chain at its end, waiting as needed).
 struct BrDescMail {      // layout of one LDS mailbox
     int word[BR_ITEM_INTS];
     int hg;
@@ -100,18 +99,20 @@ struct BrPrefetch {
     int NHG, xcc, lane;
     int qk;        // step in the queue order (global, this XCD's, the others)
     int counts;    // lane j: work units in queue j
+    int qoffs;     // lane j: index of queue j's first item
     int t_next;    // ticket drawn from the queue at step qk (lane 0), or -1
-    int stage;     // 0 ticket drawn, 1 list entry requested, 2 item requested, 9 queue ran dry
-    int idx_v, word, hg;
+    int stage;     // 0 ticket drawn, 2 item requested, 9 queue ran dry
+    int word, hg;
 
     __device__ void init(int* hdr_, const BrPlanView* pv_, int NHG_, int lane_) {
         hdr = hdr_; pv = pv_; NHG = NHG_; lane = lane_;
         xcc = br_xcc_id();
         qk = 0;
         counts = lane < BR_NQUEUES ? hdr[BR_PH_QCOUNT + lane] * NHG : 0;
+        qoffs = lane < BR_NQUEUES ? hdr[BR_PH_QOFF + lane] : 0;
         t_next = -1;
         stage = 9;
-        idx_v = word = hg = 0;
+        word = hg = 0;
     }
     __device__ void draw() {   // at the start of an item
         t_next = -1;
@@ -128,20 +129,16 @@ struct BrPrefetch {
             if (t < __builtin_amdgcn_readlane(counts, q)) {
                 const int li = t / NHG;
                 hg = t - li * NHG;
-                idx_v = pv->qlist[(size_t)q * pv->max_items + li];
-                stage = 1;
+                const int idx = __builtin_amdgcn_readlane(qoffs, q) + li;
+                word = reinterpret_cast<const int*>(pv->items + idx)[lane & (BR_ITEM_INTS - 1)];
+                stage = 2;
             } else {
                 stage = 9;
             }
-        } else if (stage == 1) {
-            const int idx = __builtin_amdgcn_readfirstlane(idx_v);
-            word = reinterpret_cast<const int*>(pv->items + idx)[lane & (BR_ITEM_INTS - 1)];
-            stage = 2;
         }
     }
     __device__ void publish(BrDescMail* mail) {   // at the end of an item
         if (stage == 0) step();
-        if (stage == 1) step();
         if (stage == 9) {
             // the queue ran dry (or nothing was drawn): look through the remaining queues now
             int qt = -1;
@@ -468,6 +465,10 @@ struct Prefill {
         }
 
         // ---- epilogue: lane (ln, lh) holds row row0+ln, dims 32d + 8(v/4) + 4lh + v%4 ----
+        // (the lane index is laundered so that the output addresses are computed here, not hoisted
+        // to the top of the item where they would have to be spilled across the key loop)
+        int lane_e = lane;
+        asm volatile("" : "+v"(lane_e));
         const float l_tot = l_run + __shfl_xor(l_run, 32);
         if (it.slot >= 0) {
             if (row0 + ln < len_m) {
@@ -508,7 +509,7 @@ struct Prefill {
                                 (long long)(qtok0 + row0) * p.so_t;
 #pragma unroll
                 for (int i = 0; i < (BR_RB * CPR) / 64; ++i) {
-                    int ch = lane + i * 64;
+                    int ch = lane_e + i * 64;
                     int row = ch / CPR, c8 = ch - row * CPR;
                     if (row0 + row < len_m) {
                         uint4 val = ld16(Es + row * SM::eRow + c8 * 8);
