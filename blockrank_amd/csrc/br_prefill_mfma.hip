@@ -248,57 +248,46 @@ struct Prefill {
     }
 
     // One wave, one 64-key tile already in LDS: S^T = K Q^T, online softmax, O^T += V^T P^T.
-    // FULL: all 64 keys are visible to every row (the common case), one straight-line block with the
-    // LDS operand reads issued several MFMAs ahead of their use.  Otherwise nkb 32-key halves are
-    // computed and keys >= lim are masked per row.
-    template <bool FULL>
+    // NKB 32-key halves are computed (the second half is skipped when no row of the wave can see it);
+    // with MASK, keys >= lim (per row: the tile's real keys and the diagonal) are excluded.  Every
+    // variant is one straight-line block with the LDS operand reads issued ahead of their use.
+    template <int NKB, bool MASK>
     static __device__ inline void compute_tile(const char* stage, const Lane& L, const bf16x8 (&qf)[D / 16], f32x16 (&o)[D / 32],
-                                               float& m_run, float& l_run, float scale_log2, int nkb, int lim, int lh) {
-        constexpr int NC = D / 16, ND = D / 32;
+                                               float& m_run, float& l_run, float scale_log2, int lim, int lh) {
+        constexpr int NC = D / 16, ND = D / 32, NR = NKB * NC;
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        f32x16 s[2];
-        if (FULL) {
-            // the two key halves alternate so that consecutive MFMAs are independent; reads run 4 ahead
+        f32x16 s[NKB];
+        {
+            // read i: half i % NKB, chunk i / NKB - the halves alternate so that consecutive MFMAs are
+            // independent; reads run 4 ahead
             bf16x8 ka[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ka[i] = read_k(stage, L, i & 1, i >> 1);
-            s[0] = zero;
-            s[1] = zero;
+            for (int i = 0; i < 4; ++i) ka[i] = read_k(stage, L, i % NKB, i / NKB);
 #pragma unroll
-            for (int i = 0; i < 2 * NC; ++i) {
+            for (int kb = 0; kb < NKB; ++kb) s[kb] = zero;
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
                 const bf16x8 a = ka[i & 3];
-                if (i + 4 < 2 * NC) ka[i & 3] = read_k(stage, L, (i + 4) & 1, (i + 4) >> 1);
-                s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[i >> 1], s[i & 1], 0, 0, 0);
+                if (i + 4 < NR) ka[i & 3] = read_k(stage, L, (i + 4) % NKB, (i + 4) / NKB);
+                s[i % NKB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[i / NKB], s[i % NKB], 0, 0, 0);
             }
-        } else {
+        }
+        // first V^T operands: their LDS latency passes under the softmax arithmetic
+        bf16x8 va[ND];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                if (kb < nkb) {
-                    f32x16 acc = zero;
+        for (int d = 0; d < ND; ++d) va[d] = read_vt(stage, L, d, 0);
+        if (MASK) {
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(read_k(stage, L, kb, c), qf[c], acc, 0, 0, 0);
-                    s[kb] = acc;
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) s[kb][v] = -INFINITY;
-                }
-            }
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     int key = kb * 32 + 16 * (v >> 3) + 8 * lh + (v & 7);
                     if (key >= lim) s[kb][v] = -INFINITY;
                 }
         }
-        // first V^T operands: their LDS latency passes under the softmax arithmetic
-        bf16x8 va[ND];
-#pragma unroll
-        for (int d = 0; d < ND; ++d) va[d] = read_vt(stage, L, d, 0);
-
         float mx = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -318,9 +307,9 @@ struct Prefill {
         }
         const float m_sub = m_run == -INFINITY ? 0.f : m_run;
         float psum = 0.f;
-        bf16x8 pf[4];
+        bf16x8 pf[2 * NKB];
 #pragma unroll
-        for (int c2 = 0; c2 < 4; ++c2) {
+        for (int c2 = 0; c2 < 2 * NKB; ++c2) {
             f32x8 t;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -331,13 +320,11 @@ struct Prefill {
         }
         l_run += psum;
 #pragma unroll
-        for (int c2 = 0; c2 < 4; ++c2) {
-            if (FULL || c2 < 2 * nkb) {
+        for (int c2 = 0; c2 < 2 * NKB; ++c2) {
 #pragma unroll
-                for (int d = 0; d < ND; ++d) {
-                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d], pf[c2], o[d], 0, 0, 0);
-                    if (c2 + 1 < 4 && (FULL || c2 + 1 < 2 * nkb)) va[d] = read_vt(stage, L, d, c2 + 1);
-                }
+            for (int d = 0; d < ND; ++d) {
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d], pf[c2], o[d], 0, 0, 0);
+                if (c2 + 1 < 2 * NKB) va[d] = read_vt(stage, L, d, c2 + 1);
             }
         }
     }
@@ -449,11 +436,13 @@ struct Prefill {
             if (!rb_active) nkb = 0;
             const bool need_mask = (cur.nvalid < nkb * 32) || (cur.self && key0 + nkb * 32 - 1 > row0);
             if (nkb == 2 && !need_mask) {
-                compute_tile<true>(stage, L, qf, o, m_run, l_run, p.scale_log2, 2, 0, lh);
+                compute_tile<2, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, 0, lh);
             } else if (nkb > 0) {
                 const int lim_causal = cur.self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
-                const int lim = need_mask ? (cur.nvalid < lim_causal ? cur.nvalid : lim_causal) : BR_BN;
-                compute_tile<false>(stage, L, qf, o, m_run, l_run, p.scale_log2, nkb, lim, lh);
+                const int lim = cur.nvalid < lim_causal ? cur.nvalid : lim_causal;
+                if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh);
+                else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh);
+                else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh);
             }
 
             if (wave == 0) pf.step();
