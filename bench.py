@@ -105,6 +105,9 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times, so that a profiler's HBM byte counters can be "
+                         "scaled against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: ranking requests are independent and this build uses a single MI355X "
@@ -140,6 +143,14 @@ def main():
         out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events)
         scores = handle.doc_scores(rows, temperature=0.05) if handle is not None else None
         return out, scores
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

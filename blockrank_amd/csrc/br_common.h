@@ -13,7 +13,7 @@
 #define BR_BN 64              // keys per key/value tile
 #define BR_RB 32              // query rows per wave (one 32x32 MFMA row block)
 #define BR_SLOTS_PER_SEQ 32   // split-KV partial slots available to one sequence's query block
-#define BR_MIN_CHUNK 4        // a split of the query block's key walk covers at least this many tiles
+#define BR_MIN_CHUNK 8        // a split of the query block's key walk covers at least this many tiles
 
 // Plan buffer (int32):
 //   [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
