@@ -128,7 +128,8 @@ def main():
     else:
         q, k, v = synthetic.random_qkv(layout, Nq, Nkv, D, dtype, dev)
     valid = layout.valid.to(dev)
-    rows = torch.tensor([[layout.H - 2, layout.H - 1]] * layout.B, dtype=torch.int32, device=dev)   # "[" and the token before it
+    R = min(16, layout.H)
+    rows16 = torch.tensor([[R - 2, R - 1]] * layout.B, dtype=torch.int32, device=dev)   # "[" and the token before it, in the last 16 positions
     module = _Module(20, Nq // Nkv)
 
     # once per forward pass: mask hook -> plan
@@ -141,7 +142,7 @@ def main():
 
     def step(events=None):
         out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events)
-        scores = handle.doc_scores(rows, temperature=0.05) if handle is not None else None
+        scores = handle.doc_scores_window(rows16, temperature=0.05) if handle is not None else None
         return out, scores
 
     if args.calibrate_copy:

@@ -17,6 +17,7 @@ from .attention import (
     blockrank_attention_forward,
     blockrank_attention_mask,
     doc_scores,
+    doc_scores_from_partials,
     last_block_logits,
     register_blockrank_attention,
     register_triton_blockrank_attention,
@@ -30,6 +31,7 @@ __all__ = [
     "blockrank_attention_forward",
     "blockrank_attention_mask",
     "doc_scores",
+    "doc_scores_from_partials",
     "last_block_logits",
     "register_blockrank_attention",
     "register_triton_blockrank_attention",

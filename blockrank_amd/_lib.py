@@ -34,6 +34,12 @@ SIGNATURES = {
     "br_prefill_fwd_events": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t, c_void_p,
                                       c_void_p, c_void_p]),
+    "br_score_partials_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "br_prefill_fwd_scores": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t,
+                                      c_int, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "br_doc_scores_from_partials": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                                            c_void_p, c_void_p, c_void_p]),
     "br_doc_scores_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "br_doc_scores": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                               c_void_p, c_void_p, c_float, c_float, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -176,14 +176,19 @@ def blockrank_attention(
     scaling: float,
     *,
     kernel_events=None,
-) -> torch.Tensor:
+    score_rows: int = 0,
+):
     """Block-sparse prefill attention.  query (B, Nq, S, D), key/value (B, Nkv, S, D) with any
     (batch, head, token) strides; block_mask a BlockMask, a (B, M, H) bool tensor, or the reference's
     (B, 1, M, H, H) additive tensor.  Returns (B, S, Nq, D) contiguous, rows of padded slots zero.
 
     Same result as sdpa_blockrank_attention_forward (blockrank_std_attention.py:503-650) on rows of
     real tokens.  kernel_events: optional pair of raw hipEvent_t handles recorded right before and
-    after the main attention kernel (see blockrank_amd.profiling)."""
+    after the main attention kernel (see blockrank_amd.profiling).
+
+    score_rows > 0 (bf16, at least one document block): the same kernel pass also leaves the per-tile
+    score partials of the query block's last score_rows positions, and the call returns
+    (out, partials); ``doc_scores_from_partials`` turns them into per-document scores."""
     if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
         block_mask = BlockMask(block_mask, query.dtype)
     bm = _as_block_mask(block_mask)
@@ -214,11 +219,54 @@ def blockrank_attention(
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         out_strides = _lib._I64x3(S * Nq * D, D, Nq * D)
         ev0, ev1 = kernel_events if kernel_events is not None else (None, None)
+        if score_rows > 0:
+            sp_bytes = lib.br_score_partials_bytes(B, Nq, M, H, score_rows)
+            part = torch.empty(max(sp_bytes // 4, 4), dtype=torch.float32, device=dev)
+            _lib.check(lib.br_prefill_fwd_scores(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
+                _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), out_strides, float(scaling),
+                _DTYPE_CODE[query.dtype], ws.data_ptr(), ws_bytes, score_rows, part.data_ptr(), sp_bytes,
+                _stream_ptr(dev), ev0, ev1))
+            return out, part
         _lib.check(lib.br_prefill_fwd_events(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
             _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), out_strides, float(scaling), _DTYPE_CODE[query.dtype],
             ws.data_ptr(), ws_bytes, _stream_ptr(dev), ev0, ev1))
     return out
+
+
+def fused_scores_supported(query: torch.Tensor, block_mask) -> bool:
+    """Whether blockrank_attention(..., score_rows=R) can produce score partials for these inputs."""
+    return query.dtype == torch.bfloat16 and block_mask.M >= 3
+
+
+def doc_scores_from_partials(partials: torch.Tensor, block_mask, rows: torch.Tensor, score_rows: int, num_heads: int,
+                             num_kv_heads: int, temperature: float = 0.05, head_reduce: str = "mean",
+                             row_reduce: str = "mean", return_probs: bool = False):
+    """Per-document scores (B, M-2) from the partials of blockrank_attention(..., score_rows=...).
+    rows: (B, R) indices 0..score_rows-1 into the last score_rows positions of the query block, as
+    losses.py:43-48 computes them.  Same value as ``doc_scores`` for those rows."""
+    bm = _as_block_mask(block_mask)
+    assert bm.M >= 3, "per-document scores need at least one document block"
+    assert head_reduce in ("mean", "sum") and row_reduce in ("mean", "sum")
+    assert rows.dim() == 2 and rows.shape[0] == bm.B, "rows must be (B, R)"
+    B, R = rows.shape
+    out_scale = 1.0 / temperature
+    if head_reduce == "mean":
+        out_scale /= num_heads
+    if row_reduce == "mean":
+        out_scale /= R
+    lib = _lib.load()
+    dev = partials.device
+    rows = rows.to(device=dev, dtype=torch.int32).contiguous()
+    with torch.cuda.device(dev):
+        plan = bm.plan(num_heads, num_kv_heads)
+        scores = torch.empty((B, bm.M - 2), dtype=torch.float32, device=dev)
+        probs = torch.empty((B, num_heads, R, bm.M - 2), dtype=torch.float32, device=dev) if return_probs else None
+        _lib.check(lib.br_doc_scores_from_partials(
+            partials.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, score_rows, B, num_heads, bm.M, bm.H,
+            float(out_scale), scores.data_ptr(), probs.data_ptr() if probs is not None else None, _stream_ptr(dev)))
+    return (scores, probs) if return_probs else scores
 
 
 class LastBlockScores:
@@ -229,9 +277,10 @@ class LastBlockScores:
     ``compute_auxiliary_attention_loss`` of this package accepts it directly; ``dense()`` produces the
     reference tensor for anything else."""
 
-    def __init__(self, query, key, block_mask: BlockMask, scaling: float, num_rows: int, scaled: bool = True):
+    def __init__(self, query, key, block_mask: BlockMask, scaling: float, num_rows: int, scaled: bool = True, partials=None):
         self.query, self.key, self.block_mask = query, key, block_mask
         self.scaling, self.R, self.scaled = float(scaling), int(num_rows), scaled
+        self.partials = partials if scaled else None    # per-tile (max, sum) pairs left by the attention kernel
         B, Nq, S, D = query.shape
         self.shape = torch.Size((B, Nq, self.R, S))
         self.device, self.dtype = query.device, query.dtype
@@ -257,6 +306,19 @@ class LastBlockScores:
         """Per-document scores for ``rows`` (B, R') positions inside the query block (0..H-1)."""
         return doc_scores(self.query, self.key, self.block_mask, rows, self.scaling if self.scaled else 1.0,
                           temperature=temperature, head_reduce=head_reduce, row_reduce=row_reduce, return_probs=return_probs)
+
+    def doc_scores_window(self, rows: torch.Tensor, temperature: float = 0.05, head_reduce: str = "mean",
+                          row_reduce: str = "mean", return_probs: bool = False):
+        """Same for ``rows`` (B, R') given as indices 0..R-1 into the handle's own R rows (the last R
+        positions of the query block).  Uses the partials the attention kernel left when there are
+        any; otherwise the stand-alone score kernels."""
+        if self.partials is not None:
+            return doc_scores_from_partials(self.partials, self.block_mask, rows, self.R, self.query.shape[1],
+                                            self.key.shape[1], temperature=temperature, head_reduce=head_reduce,
+                                            row_reduce=row_reduce, return_probs=return_probs)
+        pos = (rows + (self.block_mask.H - self.R)).to(torch.int32)
+        return self.doc_scores(pos, temperature=temperature, head_reduce=head_reduce, row_reduce=row_reduce,
+                               return_probs=return_probs)
 
 
 def _score_args(query, key, block_mask, rows):
@@ -363,21 +425,26 @@ def blockrank_attention_forward(
     if dropout > 0.0 and getattr(module, "training", False):
         warnings.warn("Dropout is not supported in kernelized BlockRank attention, ignoring dropout parameter")
 
-    out = blockrank_attention(query, key, value, bm, scaling, kernel_events=kwargs.get("kernel_events", None))
-    if bm.M == 1:
-        return out, None
-
     layers = kwargs.get("layers_to_return_scores", None)
     if layers is not None:
         layer_idx = getattr(module, "layer_idx", None)
         want = layer_idx is not None and layer_idx in layers
     else:
         want = kwargs.get("return_last_block_attn_scores", False)
-    if not want:
-        return out, None
+    want = want and bm.M > 1
     num_last = kwargs.get("num_last_queries", 16)
     R = num_last if bm.H >= num_last else bm.H
-    handle = LastBlockScores(query, key, bm, scaling, R, scaled=not kwargs.get("unscaled_scores", False))
+    scaled = not kwargs.get("unscaled_scores", False)
+    fuse = want and scaled and fused_scores_supported(query, bm) and not _env_flag("BLOCKRANK_AMD_SEPARATE_SCORES")
+
+    out = blockrank_attention(query, key, value, bm, scaling, kernel_events=kwargs.get("kernel_events", None),
+                              score_rows=R if fuse else 0)
+    partials = None
+    if fuse:
+        out, partials = out
+    if not want:
+        return out, None
+    handle = LastBlockScores(query, key, bm, scaling, R, scaled=scaled, partials=partials)
     if kwargs.get("materialize_scores", False) or _env_flag("BLOCKRANK_AMD_DENSE_SCORES"):
         return out, handle.dense()
     return out, handle

@@ -16,6 +16,8 @@ int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
                          float* probs, const long long* sq, const long long* sk, int B, int Nq, int Nkv, int M, int H, int D,
                          int R, int T, float scale, float out_scale, int dtype, hipStream_t stream);
+int br_launch_doc_scores_tiles(const float* part, const int* plan, const int* rows, float* scores, float* probs, int B, int Nq,
+                               int M, int H, int R, int Rw, float out_scale, hipStream_t stream);
 int br_launch_last_logits(const void* q, const void* k, const int* plan, const int* rows, float* logits, const long long* sq,
                           const long long* sk, int B, int Nq, int Nkv, int M, int H, int D, int R, int T, float scale,
                           float neg, int dtype, hipStream_t stream);
@@ -160,12 +162,25 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     return rows * (size_t)(D + 2) * sizeof(float);
 }
 
-int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
-                          int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                          const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
-                          void* stream, void* ev_start, void* ev_stop) {
+size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows) {
+    if (B <= 0 || Nq <= 0 || M < 3 || H <= 0 || score_rows <= 0) return 0;
+    return (size_t)B * Nq * score_rows * br_plan_tps(M, H) * 2 * sizeof(float);
+}
+
+static int prefill_impl(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                        int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
+                        void* stream, void* ev_start, void* ev_stop, int score_rows, float* score_part, size_t score_part_bytes) {
     int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
     if (rc) return rc;
+    if (score_part) {
+        if (dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "score partials come from the bf16 kernel only; use br_doc_scores");
+        if (M < 3) return fail(BR_ERR_ARG, "score partials need at least one document block (M=%d)", M);
+        if (score_rows <= 0 || score_rows > H) return fail(BR_ERR_ARG, "score_rows=%d outside 1..H=%d", score_rows, H);
+        if (!aligned16(score_part)) return fail(BR_ERR_ARG, "score_part must be 16-byte aligned");
+        const size_t sneed = br_score_partials_bytes(B, Nq, M, H, score_rows);
+        if (score_part_bytes < sneed) return fail(BR_ERR_SPACE, "score_part holds %zu bytes, %zu needed", score_part_bytes, sneed);
+    }
     if (!q || !k || !v || !out || !plan) return fail(BR_ERR_ARG, "null pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(plan) || !aligned16(workspace))
         return fail(BR_ERR_ARG, "q, k, v, out, plan and workspace must be 16-byte aligned");
@@ -192,6 +207,8 @@ int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out
     p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H;
     p.geom = g;
     p.scale_log2 = scale * 1.4426950408889634f;
+    p.score_part = score_part;
+    p.score_R = score_part ? score_rows : 0;
     int combine_grid = br_plan_max_comb(B) * g.NHG;
     if (combine_grid < B * M) combine_grid = B * M;
     if (combine_grid > 4 * n_cu) combine_grid = 4 * n_cu;
@@ -203,11 +220,42 @@ int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out
     return check_launch("prefill launch");
 }
 
+int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                          int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                          const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
+                          void* stream, void* ev_start, void* ev_stop) {
+    return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
+                        workspace, workspace_bytes, stream, ev_start, ev_stop, 0, nullptr, 0);
+}
+
 int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
                    int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                    const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
-    return br_prefill_fwd_events(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale,
-                                 dtype, workspace, workspace_bytes, stream, nullptr, nullptr);
+    return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
+                        workspace, workspace_bytes, stream, nullptr, nullptr, 0, nullptr, 0);
+}
+
+int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                          int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                          const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
+                          int score_rows, float* score_part, size_t score_part_bytes, void* stream, void* ev_start,
+                          void* ev_stop) {
+    if (!score_part) return fail(BR_ERR_ARG, "score_part must be provided");
+    return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
+                        workspace, workspace_bytes, stream, ev_start, ev_stop, score_rows, score_part, score_part_bytes);
+}
+
+int br_doc_scores_from_partials(const float* score_part, const int32_t* plan, const int32_t* rows, int R, int score_rows, int B,
+                                int Nq, int M, int H, float out_scale, float* scores, float* probs, void* stream) {
+    if (B <= 0 || Nq <= 0 || H <= 0) return fail(BR_ERR_ARG, "bad sizes B=%d Nq=%d H=%d", B, Nq, H);
+    if (M < 3) return fail(BR_ERR_ARG, "per-document scores need at least one document block (M=%d)", M);
+    if (R <= 0 || R > 16) return fail(BR_ERR_ARG, "R=%d rows not supported (1..16)", R);
+    if (score_rows <= 0 || score_rows > H) return fail(BR_ERR_ARG, "score_rows=%d outside 1..H=%d", score_rows, H);
+    if (!score_part || !plan || !rows || !scores) return fail(BR_ERR_ARG, "null pointer");
+    if (br_launch_doc_scores_tiles(score_part, plan, rows, scores, probs, B, Nq, M, H, R, score_rows, out_scale,
+                                   static_cast<hipStream_t>(stream)))
+        return fail(BR_ERR_ARG, "too many documents (%d) for the score reduction", M - 2);
+    return check_launch("score reduction launch");
 }
 
 size_t br_doc_scores_workspace_bytes(int B, int Nq, int M, int R) {

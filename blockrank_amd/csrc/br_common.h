@@ -156,6 +156,7 @@ __host__ __device__ inline int br_prev_blocks(int m, int M) {
 
 // Walk over the key/value tiles one query tile sees.  Every field is uniform across the workgroup.
 struct BrTile {
+    int flat;     // index among the sequence's earlier-block tile descriptors, -1 for the block's own tiles
     int tok0;     // token index (inside the sequence) of the tile's first key
     int kt;       // for the block's own tiles: tile index inside the block (first key is kt*BR_BN)
     int nvalid;   // real keys in the tile (1..BR_BN)
@@ -184,6 +185,7 @@ struct BrWalk {
         }
         const int kt = f - nprev, k0 = kt * BR_BN;
         if (k0 >= self_end) return 0;
+        t.flat = -1;
         t.tok0 = own_tok0 + k0;
         t.kt = kt;
         t.nvalid = self_end - k0 < BR_BN ? self_end - k0 : BR_BN;
@@ -195,6 +197,7 @@ struct BrWalk {
 
 // Descriptor of earlier-block tile i of a document (the only earlier block is the prefix).
 __device__ inline void br_prefix_tile(const BrItem& it, int i, BrTile& t) {
+    t.flat = i;
     t.tok0 = it.start0 + i * BR_BN;
     t.kt = i;
     t.nvalid = it.len0 - i * BR_BN < BR_BN ? it.len0 - i * BR_BN : BR_BN;
@@ -229,4 +232,9 @@ struct BrPrefillParams {
     int B, Nq, Nkv, M, H;
     BrGeom geom;
     float scale_log2;  // softmax scale * log2(e)
+    // Optional score partials of the query block's last score_R rows (padded positions H-score_R..H-1):
+    // [B][Nq][score_R][TPS][2] = (reference max in the log2 domain, sum of 2^(logit - max)) per earlier-block
+    // key tile, in the order of the sequence's tile descriptors.  Null: not wanted.
+    float* score_part;
+    int score_R;
 };

@@ -253,7 +253,7 @@ struct Prefill {
     // variant is one straight-line block with the LDS operand reads issued ahead of their use.
     template <int NKB, bool MASK>
     static __device__ inline void compute_tile(const char* stage, const Lane& L, const bf16x8 (&qf)[D / 16], f32x16 (&o)[D / 32],
-                                               float& m_run, float& l_run, float scale_log2, int lim, int lh) {
+                                               float& m_run, float& l_run, float scale_log2, int lim, int lh, float& psum_out) {
         constexpr int NC = D / 16, ND = D / 32, NR = NKB * NC;
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         f32x16 s[NKB];
@@ -319,6 +319,7 @@ struct Prefill {
             pf[c2] = __builtin_convertvector(t, bf16x8);
         }
         l_run += psum;
+        psum_out = psum;
 #pragma unroll
         for (int c2 = 0; c2 < 2 * NKB; ++c2) {
 #pragma unroll
@@ -357,6 +358,9 @@ struct Prefill {
         walk.init(it, self_end, p.H);
         const int2* tiles_b = pv.tiles + (size_t)b * pv.tps;
         const bool table = it.pe > 1;
+        // only query-block items of a sequence with documents emit score partials, for document tiles
+        const bool emit_scores = p.score_part != nullptr && table && m == p.M - 1;
+        const int first_doc_tile = (it.len0 + BR_BN - 1) / BR_BN;
         int dbase = it.f_lo;
         int2 dreg = make_int2(0, 0);
         if (table && dbase + lane < it.nprev) dreg = tiles_b[dbase + lane];
@@ -373,6 +377,7 @@ struct Prefill {
                         dreg = dbase + lane < it.nprev ? tiles_b[dbase + lane] : make_int2(0, 0);
                         asm volatile("" : "+v"(dreg.x), "+v"(dreg.y));   // wait here, not at every later use
                     }
+                    t.flat = pi;
                     t.tok0 = __builtin_amdgcn_readlane(dreg.x, pi - dbase);
                     t.nvalid = __builtin_amdgcn_readlane(dreg.y, pi - dbase);
                     t.kt = 0;
@@ -435,14 +440,25 @@ struct Prefill {
             }
             if (!rb_active) nkb = 0;
             const bool need_mask = (cur.nvalid < nkb * 32) || (cur.self && key0 + nkb * 32 - 1 > row0);
+            float psum = 0.f;
             if (nkb == 2 && !need_mask) {
-                compute_tile<2, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, 0, lh);
+                compute_tile<2, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, 0, lh, psum);
             } else if (nkb > 0) {
                 const int lim_causal = cur.self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
                 const int lim = cur.nvalid < lim_causal ? cur.nvalid : lim_causal;
-                if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh);
-                else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh);
-                else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh);
+                if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
+                else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
+                else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
+            }
+            // Score partials: this tile's probability mass (against the running max) for the query block's
+            // last rows, per head - everything the per-document scores need, with no second pass over K.
+            if (emit_scores && nkb > 0 && cur.flat >= first_doc_tile) {
+                const float tot = psum + __shfl_xor(psum, 32);
+                const int r16 = it.start_m + row0 + ln - (p.H - p.score_R);
+                if (lh == 0 && r16 >= 0 && row0 + ln < len_m) {
+                    float2 ms = make_float2(m_run == -INFINITY ? 0.f : m_run, tot);
+                    *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + cur.flat) * 2) = ms;
+                }
             }
 
             if (wave == 0) pf.step();

@@ -226,6 +226,124 @@ __global__ __launch_bounds__(256) void br_doc_final_kernel(BrScoreParams p) {
     }
 }
 
+// Per-document scores from the per-tile partials the prefill kernel leaves for the query block's last
+// Rw rows: part[b][n][r][tile] = (max, sum of 2^(logit - max)) over that tile's real keys, tiles in the
+// order of the sequence's tile descriptors (document d owns tiles tbase[d+1] .. + ceil(len/64)).
+// One workgroup per sequence; every wave takes (head, row) pairs round robin, a lane takes a
+// document: joint normalisation over all documents, then the per-document sums are added into the
+// wave's own accumulator row in LDS; the rows are added up in a fixed order at the end.
+struct BrTileScoreParams {
+    const float* part;
+    const int* plan;
+    const int* rows;        // (B, R) indices into the last Rw positions of the query block
+    float* scores;          // (B, docs)
+    float* probs;           // optional (B, Nq, R, docs)
+    int B, Nq, M, H, R, Rw;
+    float out_scale;
+};
+
+__global__ __launch_bounds__(1024) void br_doc_final_tiles_kernel(BrTileScoreParams p) {
+    extern __shared__ float dyn[];      // [nwaves][docs]
+    const int docs = p.M - 2;
+    const int b = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+    const int* start = p.plan + br_plan_off_start();
+    const int* len = p.plan + br_plan_off_len(p.B, p.M);
+    const int* tbase = p.plan + br_plan_off_tbase(p.B, p.M);
+    const int tps = br_plan_tps(p.M, p.H);
+    const int NR = p.Nq * p.R;
+    const int st_q = start[b * p.M + p.M - 1], len_q = len[b * p.M + p.M - 1];
+    float* mine = dyn + wave * docs;
+    for (int d = lane; d < docs; d += 64) mine[d] = 0.f;
+    const float uniform = 1.f / (float)docs;
+    const bool small = docs <= 64 && p.H <= 8 * BR_BN;   // one document per lane, its tiles in registers
+    int t0 = 0, nt = 0;
+    if (small && lane < docs) {
+        t0 = tbase[b * p.M + lane + 1];
+        nt = (len[b * p.M + lane + 1] + BR_BN - 1) / BR_BN;
+    }
+    for (int j = wave; j < NR; j += nwaves) {
+        const int n = j / p.R, r = j - n * p.R;
+        int r16 = p.rows[b * p.R + r];
+        r16 = r16 < 0 ? 0 : (r16 >= p.Rw ? p.Rw - 1 : r16);
+        const int pos = p.H - p.Rw + r16;
+        const bool row_ok = pos >= st_q && pos < st_q + len_q;
+        const float2* base = reinterpret_cast<const float2*>(p.part) + (((long long)b * p.Nq + n) * p.Rw + r16) * tps;
+        float* pr_out = p.probs ? p.probs + ((long long)b * NR + j) * docs : nullptr;
+        if (small) {
+            float2 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = (row_ok && i < nt) ? base[t0 + i] : make_float2(-INFINITY, 0.f);
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) mx = fmaxf(mx, v[i].x);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            float sd = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (v[i].x != -INFINITY) sd += v[i].y * __builtin_amdgcn_exp2f(v[i].x - mx);
+            float den = sd;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
+            if (lane < docs) {
+                const float pr = den > 0.f ? sd / den : uniform;
+                if (pr_out) pr_out[lane] = pr;
+                mine[lane] += pr;
+            }
+        } else {
+            float mx = -INFINITY;
+            if (row_ok)
+                for (int d = lane; d < docs; d += 64) {
+                    const int f0 = tbase[b * p.M + d + 1], f1 = f0 + (len[b * p.M + d + 1] + BR_BN - 1) / BR_BN;
+                    for (int f = f0; f < f1; ++f) mx = fmaxf(mx, base[f].x);
+                }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            float den = 0.f;
+            if (mx != -INFINITY)
+                for (int d = lane; d < docs; d += 64) {
+                    const int f0 = tbase[b * p.M + d + 1], f1 = f0 + (len[b * p.M + d + 1] + BR_BN - 1) / BR_BN;
+                    float sd = 0.f;
+                    for (int f = f0; f < f1; ++f) {
+                        const float2 ms = base[f];
+                        sd += ms.y * __builtin_amdgcn_exp2f(ms.x - mx);
+                    }
+                    den += sd;
+                    if (pr_out) pr_out[d] = sd;       // unnormalised for now, only this lane touches it
+                }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
+            const float inv = den > 0.f ? 1.f / den : 0.f;
+            for (int d = lane; d < docs; d += 64) {
+                float pr = uniform;
+                if (inv != 0.f) {
+                    float sd;
+                    if (pr_out) {
+                        sd = pr_out[d];
+                    } else {
+                        const int f0 = tbase[b * p.M + d + 1], f1 = f0 + (len[b * p.M + d + 1] + BR_BN - 1) / BR_BN;
+                        sd = 0.f;
+                        for (int f = f0; f < f1; ++f) {
+                            const float2 ms = base[f];
+                            sd += ms.y * __builtin_amdgcn_exp2f(ms.x - mx);
+                        }
+                    }
+                    pr = sd * inv;
+                }
+                if (pr_out) pr_out[d] = pr;
+                mine[d] += pr;
+            }
+        }
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < docs; d += blockDim.x) {
+        float acc = 0.f;
+        for (int w = 0; w < nwaves; ++w) acc += dyn[w * docs + d];
+        p.scores[(long long)b * docs + d] = acc * p.out_scale;
+    }
+}
+
 // s_last[b, n, r, key] = scale * q.k + (0 if the row may see the key else NEG), every key slot of
 // the padded sequence included (blockrank_std_attention.py:639-645 with the eager scaling of :154).
 template <typename T, int D>
@@ -320,3 +438,17 @@ int br_launch_last_logits(const void* q, const void* k, const int* plan, const i
         hipLaunchKernelGGL((br_last_logits_kernel<__bf16, 128>), grid, dim3(256), sh, stream, p);
     return 0;
 }
+
+int br_launch_doc_scores_tiles(const float* part, const int* plan, const int* rows, float* scores, float* probs, int B, int Nq,
+                               int M, int H, int R, int Rw, float out_scale, hipStream_t stream) {
+    BrTileScoreParams p;
+    p.part = part; p.plan = plan; p.rows = rows; p.scores = scores; p.probs = probs;
+    p.B = B; p.Nq = Nq; p.M = M; p.H = H; p.R = R; p.Rw = Rw; p.out_scale = out_scale;
+    const int docs = M - 2;
+    int nwaves = 16;
+    while (nwaves > 1 && (size_t)nwaves * docs * sizeof(float) > 48 * 1024) nwaves >>= 1;
+    if ((size_t)nwaves * docs * sizeof(float) > 60 * 1024) return 1;
+    hipLaunchKernelGGL(br_doc_final_tiles_kernel, dim3(B), dim3(nwaves * 64), (size_t)nwaves * docs * sizeof(float), stream, p);
+    return 0;
+}
+

@@ -58,8 +58,7 @@ def compute_auxiliary_attention_loss(
     assert MH == M * H, "Attention scores last dimension must match M*H"
     rows = bracket_rows(labels, h1)                                  # (B, 2) in [0, h1)
     if isinstance(attention_scores, LastBlockScores):
-        pos = (rows + (H - h1)).to(torch.int32)                      # positions inside the query block
-        logits = attention_scores.doc_scores(pos, temperature=temperature)
+        logits = attention_scores.doc_scores_window(rows, temperature=temperature)
     else:
         x = attention_scores.take_along_dim(rows[:, None, :, None], dim=2)[..., H:-H]
         p = F.softmax(x, dim=-1).reshape(B, N, -1, M - 2, H)

@@ -86,6 +86,32 @@ int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out
                           const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype,
                           void* workspace, size_t workspace_bytes, void* stream, void* ev_start, void* ev_stop);
 
+/* Bytes of the score-partials buffer of br_prefill_fwd_scores. */
+size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows);
+
+/* br_prefill_fwd_events that, in the same pass, leaves what the per-document scores of the query
+ * block's last score_rows positions (H-score_rows .. H-1) need: for every head, such row and
+ * earlier-block key tile the pair (max, sum of exp) of the row's logits over the tile, in score_part.
+ * This is the reference's "attention + s_last in one call" (blockrank_std_attention.py:623-645;
+ * triton_blockrank_attention_forward with return_last_block_scores,
+ * blockrank_triton_kernel_attention.py:858-881) without the second pass over K; the reference uses
+ * score_rows = 16.  bf16 only (BR_DTYPE_F32 callers use br_doc_scores).  score_part needs no
+ * initialisation; it is consumed by br_doc_scores_from_partials with the same plan. */
+int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
+                          int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
+                          const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype,
+                          void* workspace, size_t workspace_bytes, int score_rows, float* score_part,
+                          size_t score_part_bytes, void* stream, void* ev_start, void* ev_stop);
+
+/* Per-document relevance from the partials of br_prefill_fwd_scores: compute_auxiliary_attention_loss(
+ * answer_ids=None, return_logits=True) (src/blockrank/losses.py:37-78).
+ *   rows: (B, R) int32 indices 0..score_rows-1 into the last score_rows positions of the query block
+ *   (what losses.py:43-48 computes from the labels); R <= 16.  scores, probs, out_scale as in
+ *   br_doc_scores. */
+int br_doc_scores_from_partials(const float* score_part, const int32_t* plan, const int32_t* rows, int R,
+                                int score_rows, int B, int Nq, int M, int H, float out_scale, float* scores,
+                                float* probs, void* stream);
+
 /* Bytes of scratch br_doc_scores needs. */
 size_t br_doc_scores_workspace_bytes(int B, int Nq, int M, int R);
 
