@@ -423,6 +423,14 @@ struct Prefill {
         int bufi = 0;
 
         while (have) {
+            // The tile descriptors are small stack objects, i.e. scratch memory, and a scratch load
+            // waits for every vector memory operation issued before it - the next tile's DMA included.
+            // So everything that reads the current descriptor happens here, before that DMA is issued
+            // (the DMA asm is a compiler barrier for memory accesses), and only values stay live.
+            int c_nvalid = cur.nvalid, c_kt = cur.kt, c_self = cur.self, c_flat = cur.flat;
+            // (the compiler places its wait for a load at the first use of the value; the empty asm is
+            // such a use, so the wait lands here and not behind the DMA it cannot see)
+            asm volatile("" : "+v"(c_nvalid), "+v"(c_kt), "+v"(c_self), "+v"(c_flat));
             const bool have_next = fetch(nxt);
             if (have_next)
                 issue_tile(L, wave, kbase + (long long)nxt.tok0 * p.sk_t, vbase + (long long)nxt.tok0 * p.sv_t, sk_bytes, sv_bytes,
@@ -431,33 +439,33 @@ struct Prefill {
 
             // 32-key halves of the tile this wave needs: limited by the real keys in the tile and, on
             // the block's own keys, by the diagonal (last row of the wave is row0 + 31).
-            int nkb = (cur.nvalid + 31) >> 5;
-            const int key0 = cur.kt * BR_BN;               // valid-relative position of the tile's first key
-            if (cur.self) {
+            int nkb = (c_nvalid + 31) >> 5;
+            const int key0 = c_kt * BR_BN;                 // valid-relative position of the tile's first key
+            if (c_self) {
                 int vis = row0 + BR_RB - key0;             // keys [0, vis) of the tile are visible to some row
                 int c = vis <= 0 ? 0 : (vis + 31) >> 5;
                 nkb = c < nkb ? c : nkb;
             }
             if (!rb_active) nkb = 0;
-            const bool need_mask = (cur.nvalid < nkb * 32) || (cur.self && key0 + nkb * 32 - 1 > row0);
+            const bool need_mask = (c_nvalid < nkb * 32) || (c_self && key0 + nkb * 32 - 1 > row0);
             float psum = 0.f;
             if (nkb == 2 && !need_mask) {
                 compute_tile<2, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, 0, lh, psum);
             } else if (nkb > 0) {
-                const int lim_causal = cur.self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
-                const int lim = cur.nvalid < lim_causal ? cur.nvalid : lim_causal;
+                const int lim_causal = c_self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
+                const int lim = c_nvalid < lim_causal ? c_nvalid : lim_causal;
                 if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
                 else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
                 else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
             }
             // Score partials: this tile's probability mass (against the running max) for the query block's
             // last rows, per head - everything the per-document scores need, with no second pass over K.
-            if (emit_scores && nkb > 0 && cur.flat >= first_doc_tile) {
+            if (emit_scores && nkb > 0 && c_flat >= first_doc_tile) {
                 const float tot = psum + __shfl_xor(psum, 32);
                 const int r16 = it.start_m + row0 + ln - (p.H - p.score_R);
                 if (lh == 0 && r16 >= 0 && row0 + ln < len_m) {
                     float2 ms = make_float2(m_run == -INFINITY ? 0.f : m_run, tot);
-                    *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + cur.flat) * 2) = ms;
+                    *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + c_flat) * 2) = ms;
                 }
             }
 
