@@ -202,8 +202,11 @@ struct Prefill {
     }
 
     // Start the DMA of one K/V tile into a stage.  kt / vt point at the tile's first row (uniform).
-    static __device__ inline void issue_tile(const Lane& L, int wave, const __bf16* kt, const __bf16* vt, int sk_bytes, int sv_bytes,
-                                             int nvalid, unsigned stage_lds) {
+    // lane_l is the lane index as an opaque value of the current loop iteration: the row arithmetic of
+    // the partial-tile path is then redone where it is needed (it is rare) instead of being kept in
+    // registers across the whole key loop.
+    static __device__ inline void issue_tile(const Lane& L, int wave, int lane_l, const __bf16* kt, const __bf16* vt, int sk_bytes,
+                                             int sv_bytes, int nvalid, unsigned stage_lds) {
         if (nvalid == BR_BN) {
 #pragma unroll
             for (int j = 0; j < JK; ++j) {
@@ -225,10 +228,17 @@ struct Prefill {
             for (int j = 0; j < JK; ++j) {
                 const int q = wave + NW * j;
                 if (NI % NW == 0 || q < NI) {
-                    const int ko = UNIFORM_STEP ? L.koff[0] + j * STEP_ROWS * sk_bytes : L.koff[j];
-                    const int vo = UNIFORM_STEP ? L.voff[0] + j * STEP_ROWS * sv_bytes : L.voff[j];
-                    if (ko < nvalid * sk_bytes) dma16(kt, ko, stage_lds + q * 1024);
-                    if (vo < nvalid * sv_bytes) dma16(vt, vo, stage_lds + SM::kBytes + q * 1024);
+                    const int prow = (q * 64 + lane_l) / CPR;                   // V row of this piece
+                    const int kkey = (prow & 32) | swap23(prow & 31);          // K row of this piece
+                    if (UNIFORM_STEP) {
+                        if (kkey < nvalid)
+                            dma16(reinterpret_cast<const char*>(kt) + j * STEP_ROWS * sk_bytes, L.koff[0], stage_lds + q * 1024);
+                        if (prow < nvalid)
+                            dma16(reinterpret_cast<const char*>(vt) + j * STEP_ROWS * sv_bytes, L.voff[0], stage_lds + SM::kBytes + q * 1024);
+                    } else {
+                        if (kkey < nvalid) dma16(kt, L.koff[j], stage_lds + q * 1024);
+                        if (prow < nvalid) dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
+                    }
                 }
             }
         }
@@ -351,45 +361,55 @@ struct Prefill {
         const __bf16* kbase = reinterpret_cast<const __bf16*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h;
         const __bf16* vbase = reinterpret_cast<const __bf16*>(p.v) + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
 
-        // The walk needs no memory lookups inside the loop: a document's only earlier block is the
-        // prefix (described by the item itself); a query-block item keeps the descriptors of its
-        // earlier-block tiles in lane registers (lane i = tile dbase + i) and reads them with readlane.
-        BrWalk walk;
-        walk.init(it, self_end, p.H);
+        // The walk over the item's key tiles needs no memory lookups inside the loop: a document's only
+        // earlier block is the prefix (described by the item itself); a query-block item keeps the
+        // descriptors of its earlier-block tiles in lane registers (lane i = tile dbase + i) and reads
+        // them with readlane.  Every quantity is a scalar computed with selects (no tile structs: they
+        // would end up in scratch memory, and a scratch load waits for the tile DMAs in flight).
         const int2* tiles_b = pv.tiles + (size_t)b * pv.tps;
         const bool table = it.pe > 1;
         // only query-block items of a sequence with documents emit score partials, for document tiles
         const bool emit_scores = p.score_part != nullptr && table && m == p.M - 1;
         const int first_doc_tile = (it.len0 + BR_BN - 1) / BR_BN;
+        const int nprev = it.nprev;
+        const int f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
+        const int own_tok0 = m * p.H + it.start_m;
+        int wf = it.f_lo;                                  // next tile of the walk
         int dbase = it.f_lo;
         int2 dreg = make_int2(0, 0);
-        if (table && dbase + lane < it.nprev) dreg = tiles_b[dbase + lane];
-        auto fetch = [&](BrTile& t) -> bool {
-            int pi = 0;
-            const int r = walk.next(t, &pi);
-            if (r == 0) return false;
-            if (r == 1) {
-                if (!table) {
-                    br_prefix_tile(it, pi, t);
-                } else {
-                    if (pi - dbase >= 64) {
-                        dbase = pi;
-                        dreg = dbase + lane < it.nprev ? tiles_b[dbase + lane] : make_int2(0, 0);
-                        asm volatile("" : "+v"(dreg.x), "+v"(dreg.y));   // wait here, not at every later use
-                    }
-                    t.flat = pi;
-                    t.tok0 = __builtin_amdgcn_readlane(dreg.x, pi - dbase);
-                    t.nvalid = __builtin_amdgcn_readlane(dreg.y, pi - dbase);
-                    t.kt = 0;
-                    t.self = 0;
-                }
+        if (table && dbase + lane < nprev) dreg = tiles_b[dbase + lane];
+        // tile state: index in the walk (earlier-block tiles come first, f < nprev; then the block's
+        // own tiles), first token, real keys
+        int c_f = 0, c_tok0 = 0, c_nvalid = 0;
+        int n_f = 0, n_tok0 = 0, n_nvalid = 0;
+        auto fetch = [&]() -> bool {
+            const int f = wf;
+            const bool prev = f < nprev;
+            const int k0 = (f - nprev) * BR_BN;
+            if (f >= f_end || (!prev && k0 >= self_end)) return false;
+            if (prev && table && f - dbase >= 64) {
+                dbase = f;
+                dreg = dbase + lane < nprev ? tiles_b[dbase + lane] : make_int2(0, 0);
+                asm volatile("" : "+v"(dreg.x), "+v"(dreg.y));   // wait here, not at every later use
             }
+            const int li = (prev && table) ? f - dbase : 0;
+            const int t_tok0 = __builtin_amdgcn_readlane(dreg.x, li), t_nv = __builtin_amdgcn_readlane(dreg.y, li);
+            const int p_nv = it.len0 - f * BR_BN < BR_BN ? it.len0 - f * BR_BN : BR_BN;
+            const int o_nv = self_end - k0 < BR_BN ? self_end - k0 : BR_BN;
+            n_f = f;
+            n_tok0 = prev ? (table ? t_tok0 : it.start0 + f * BR_BN) : own_tok0 + k0;
+            n_nvalid = prev ? (table ? t_nv : p_nv) : o_nv;
+            wf = f + 1;
             return true;
         };
-        BrTile cur, nxt;
-        bool have = fetch(cur);
-        if (have)
-            issue_tile(L, wave, kbase + (long long)cur.tok0 * p.sk_t, vbase + (long long)cur.tok0 * p.sv_t, sk_bytes, sv_bytes, cur.nvalid, smem_lds);
+        bool have = fetch();
+        c_f = n_f; c_tok0 = n_tok0; c_nvalid = n_nvalid;
+        if (have) {
+            int lane_l = lane;
+            asm volatile("" : "+v"(lane_l));
+            issue_tile(L, wave, lane_l, kbase + (long long)c_tok0 * p.sk_t, vbase + (long long)c_tok0 * p.sv_t, sk_bytes, sv_bytes, c_nvalid,
+                       smem_lds);
+        }
 
         // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.
         bf16x8 qf[D / 16];
@@ -423,49 +443,51 @@ struct Prefill {
         int bufi = 0;
 
         while (have) {
-            // The tile descriptors are small stack objects, i.e. scratch memory, and a scratch load
-            // waits for every vector memory operation issued before it - the next tile's DMA included.
-            // So everything that reads the current descriptor happens here, before that DMA is issued
-            // (the DMA asm is a compiler barrier for memory accesses), and only values stay live.
-            int c_nvalid = cur.nvalid, c_kt = cur.kt, c_self = cur.self, c_flat = cur.flat;
-            // (the compiler places its wait for a load at the first use of the value; the empty asm is
-            // such a use, so the wait lands here and not behind the DMA it cannot see)
-            asm volatile("" : "+v"(c_nvalid), "+v"(c_kt), "+v"(c_self), "+v"(c_flat));
-            const bool have_next = fetch(nxt);
+            // the lane index as a value the compiler cannot trace back: what the rare paths below derive
+            // from it (partial tiles, score partials) is computed there, not kept in registers
+            int lane_l = lane;
+            asm volatile("" : "+v"(lane_l));
+            const bool have_next = fetch();
             if (have_next)
-                issue_tile(L, wave, kbase + (long long)nxt.tok0 * p.sk_t, vbase + (long long)nxt.tok0 * p.sv_t, sk_bytes, sv_bytes,
-                           nxt.nvalid, smem_lds + (bufi ^ 1) * SM::stageBytes);
+                issue_tile(L, wave, lane_l, kbase + (long long)n_tok0 * p.sk_t, vbase + (long long)n_tok0 * p.sv_t, sk_bytes, sv_bytes,
+                           n_nvalid, smem_lds + (bufi ^ 1) * SM::stageBytes);
             const char* stage = smem + bufi * SM::stageBytes;
 
             // 32-key halves of the tile this wave needs: limited by the real keys in the tile and, on
             // the block's own keys, by the diagonal (last row of the wave is row0 + 31).
-            int nkb = (c_nvalid + 31) >> 5;
-            const int key0 = c_kt * BR_BN;                 // valid-relative position of the tile's first key
+            // (the tile quantities are handed to the arithmetic below as per-lane values: with scalar ones
+            // the compiler's code for the four tile variants needs far more registers than there are)
+            int v_nvalid = c_nvalid, v_f = c_f;
+            asm volatile("" : "+v"(v_nvalid), "+v"(v_f));
+            int nkb = (v_nvalid + 31) >> 5;
+            const bool c_self = v_f >= nprev;              // the block's own keys: the causal rule applies
+            const int key0 = (v_f - nprev) * BR_BN;        // then: position of the tile's first key in the block
             if (c_self) {
                 int vis = row0 + BR_RB - key0;             // keys [0, vis) of the tile are visible to some row
                 int c = vis <= 0 ? 0 : (vis + 31) >> 5;
                 nkb = c < nkb ? c : nkb;
             }
             if (!rb_active) nkb = 0;
-            const bool need_mask = (c_nvalid < nkb * 32) || (c_self && key0 + nkb * 32 - 1 > row0);
+            const bool need_mask = (v_nvalid < nkb * 32) || (c_self && key0 + nkb * 32 - 1 > row0);
             float psum = 0.f;
             if (nkb == 2 && !need_mask) {
                 compute_tile<2, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, 0, lh, psum);
             } else if (nkb > 0) {
                 const int lim_causal = c_self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
-                const int lim = c_nvalid < lim_causal ? c_nvalid : lim_causal;
+                const int lim = v_nvalid < lim_causal ? v_nvalid : lim_causal;
                 if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
                 else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
                 else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
             }
             // Score partials: this tile's probability mass (against the running max) for the query block's
             // last rows, per head - everything the per-document scores need, with no second pass over K.
-            if (emit_scores && nkb > 0 && c_flat >= first_doc_tile) {
+            if (emit_scores && nkb > 0 && !c_self && c_f >= first_doc_tile) {
                 const float tot = psum + __shfl_xor(psum, 32);
-                const int r16 = it.start_m + row0 + ln - (p.H - p.score_R);
-                if (lh == 0 && r16 >= 0 && row0 + ln < len_m) {
+                const int ln_l = lane_l & 31;
+                const int r16 = it.start_m + row0 + ln_l - (p.H - p.score_R);
+                if (lane_l < 32 && r16 >= 0 && row0 + ln_l < len_m) {
                     float2 ms = make_float2(m_run == -INFINITY ? 0.f : m_run, tot);
-                    *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + c_flat) * 2) = ms;
+                    *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + c_f) * 2) = ms;
                 }
             }
 
@@ -473,7 +495,7 @@ struct Prefill {
             vm_wait_all();
             __syncthreads();
             bufi ^= 1;
-            cur = nxt;
+            c_f = n_f; c_tok0 = n_tok0; c_nvalid = n_nvalid;
             have = have_next;
         }
 
