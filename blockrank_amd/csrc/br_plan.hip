@@ -120,61 +120,62 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     }
     __syncthreads();
 
-    // Pass 1: how many items each queue gets, so that the items array can be laid out queue by queue.
-    int qoff[BR_NQUEUES];
-    {
-        int qtot[BR_NQUEUES];
-#pragma unroll
-        for (int g = 0; g < BR_NQUEUES; ++g) qtot[g] = 0;
-        for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
-            const int p = p0 + tid;
-            int n_items = 0, myq = -1;
-            if (p < BM) {
-                const int b = p / M, jj = p - b * M;
-                const int m = jj == 0 ? M - 1 : jj - 1;
-                const int L = len[b * M + m];
-                const int nq = ceil_div(L, T);
-                if (jj == 0) {
-                    myq = BR_GLOBAL_QUEUE;
-                    const int pt = M > 1 ? prev_tiles[b] : 0;
-                    int ns_cap = nq > 0 ? BR_SLOTS_PER_SEQ / nq : 1;
-                    ns_cap = ns_cap < 1 ? 1 : ns_cap;
-                    for (int tt = 0; tt < nq; ++tt) {
-                        int e = (tt + 1) * T < L ? (tt + 1) * T : L;
-                        n_items += splits_for(pt + ceil_div(e, BR_BN), ns_cap);
-                    }
-                } else {
-                    myq = (b * (M - 1) + m) & 7;
-                    n_items = nq;
+    // Work distribution.  The query-block items (long walks, split) form the global queue, drained
+    // first.  All other items keep their natural order (sequence, block, query tile) and that list is
+    // cut into eight contiguous runs of equal estimated work, one per XCD queue: an XCD then works on
+    // a few adjacent blocks at a time (their K/V stay in its L2), and the runs end together, so that
+    // no workgroup has to go looking for work in other queues at the end of the kernel (polling the
+    // ticket counters there slows the memory accesses of every workgroup still working).
+    // Estimated work of an item: its key tiles plus a constant for set-up and epilogue.
+    constexpr int kItemOverhead = 2;
+    auto item_weight = [&](int nprev_t, int tt, int L) {
+        int e = (tt + 1) * T < L ? (tt + 1) * T : L;
+        return nprev_t + ceil_div(e, BR_BN) + kItemOverhead;
+    };
+    __shared__ int s_qfirst[8];
+    if (tid < 8) s_qfirst[tid] = 0x7fffffff;
+
+    // Pass 1: number of global-queue items and total weight of the others.
+    int n_glob_total = 0, n_x_total = 0;
+    long long w_total = 0;
+    for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
+        const int p = p0 + tid;
+        int n_glob = 0, n_x = 0, w_pair = 0;
+        if (p < BM) {
+            const int b = p / M, jj = p - b * M;
+            const int m = jj == 0 ? M - 1 : jj - 1;
+            const int L = len[b * M + m];
+            const int nq = ceil_div(L, T);
+            if (jj == 0) {
+                const int pt = M > 1 ? prev_tiles[b] : 0;
+                int ns_cap = nq > 0 ? BR_SLOTS_PER_SEQ / nq : 1;
+                ns_cap = ns_cap < 1 ? 1 : ns_cap;
+                for (int tt = 0; tt < nq; ++tt) {
+                    int e = (tt + 1) * T < L ? (tt + 1) * T : L;
+                    n_glob += splits_for(pt + ceil_div(e, BR_BN), ns_cap);
                 }
-            }
-#pragma unroll
-            for (int g = 0; g < BR_NQUEUES; ++g) {
-                int tot_g;
-                block_exclusive_scan(myq == g ? n_items : 0, sh, &tot_g);
-                qtot[g] += tot_g;
+            } else {
+                n_x = nq;
+                const int npt = br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0;
+                for (int tt = 0; tt < nq; ++tt) w_pair += item_weight(npt, tt, L);
             }
         }
-        // the global queue first, then the XCD queues
-        int c = 0;
-        qoff[BR_GLOBAL_QUEUE] = c;
-        c += qtot[BR_GLOBAL_QUEUE];
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
-            qoff[g] = c;
-            c += qtot[g];
-        }
+        int tot;
+        block_exclusive_scan(n_glob, sh, &tot);
+        n_glob_total += tot;
+        block_exclusive_scan(n_x, sh, &tot);
+        n_x_total += tot;
+        block_exclusive_scan(w_pair, sh, &tot);
+        w_total += tot;
     }
 
     // Pass 2: pairs (sequence, block) are visited sequence by sequence, the query block first.
-    int base_items = 0, base_comb = 0;
-    int qbase[BR_NQUEUES];
-#pragma unroll
-    for (int g = 0; g < BR_NQUEUES; ++g) qbase[g] = 0;
+    int base_glob = 0, base_x = n_glob_total, base_comb = 0;
+    long long base_w = 0;
     for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
         const int p = p0 + tid;
-        int n_items = 0, n_comb = 0, myq = -1;
-        int b = 0, m = 0, L = 0, nq = 0, ns_cap = 1, pt = 0;
+        int n_glob = 0, n_x = 0, n_comb = 0, w_pair = 0;
+        int b = 0, m = 0, L = 0, nq = 0, ns_cap = 1, pt = 0, npt = 0;
         bool is_last = false;
         if (p < BM) {
             b = p / M;
@@ -184,52 +185,51 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             L = len[b * M + m];
             nq = ceil_div(L, T);
             if (is_last) {
-                myq = BR_GLOBAL_QUEUE;
                 pt = M > 1 ? prev_tiles[b] : 0;
                 ns_cap = nq > 0 ? BR_SLOTS_PER_SEQ / nq : 1;
                 ns_cap = ns_cap < 1 ? 1 : ns_cap;
                 for (int tt = 0; tt < nq; ++tt) {
                     int e = (tt + 1) * T < L ? (tt + 1) * T : L;
                     int ns = splits_for(pt + ceil_div(e, BR_BN), ns_cap);
-                    n_items += ns;
+                    n_glob += ns;
                     n_comb += ns > 1;
                 }
             } else {
-                myq = (b * (M - 1) + m) & 7;
-                n_items = nq;
+                n_x = nq;
+                npt = br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0;
+                for (int tt = 0; tt < nq; ++tt) w_pair += item_weight(npt, tt, L);
             }
         }
-        int tot_i, tot_c;
-        block_exclusive_scan(n_items, sh, &tot_i);
+        int tot_g, tot_x, tot_c, tot_w;
+        int off_g = base_glob + block_exclusive_scan(n_glob, sh, &tot_g);
+        int off_x = base_x + block_exclusive_scan(n_x, sh, &tot_x);
         int off_c = base_comb + block_exclusive_scan(n_comb, sh, &tot_c);
-        base_items += tot_i;
+        long long off_w = base_w + block_exclusive_scan(w_pair, sh, &tot_w);
+        base_glob += tot_g;
+        base_x += tot_x;
         base_comb += tot_c;
-        // position of this pair's items in its queue's list
-        int qpos = 0;
-#pragma unroll
-        for (int g = 0; g < BR_NQUEUES; ++g) {
-            int tot_g;
-            int r = block_exclusive_scan(myq == g ? n_items : 0, sh, &tot_g);
-            if (myq == g) qpos = qoff[g] + qbase[g] + r;
-            qbase[g] += tot_g;
-        }
+        base_w += tot_w;
         if (p < BM) {
-            int off_i = qpos;     // this pair's items sit together inside its queue's run
             const int pe = br_prev_blocks(m, M);
             BrItem it;
             it.b = b; it.m = m; it.pe = pe;
             it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
             it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
             if (!is_last) {
-                it.nprev = pe > 0 ? ceil_div(it.len0, BR_BN) : 0;
+                it.nprev = npt;
                 for (int tt = 0; tt < nq; ++tt) {
                     it.t0 = tt * T; it.f_lo = 0;
                     it.ntiles = 0x7fffffff; it.slot = -1;
-                    items[off_i + tt] = it;
+                    items[off_x + tt] = it;
+                    int q = w_total > 0 ? (int)(off_w * 8 / w_total) : 0;
+                    q = q > 7 ? 7 : q;
+                    atomicMin(&s_qfirst[q], off_x + tt);
+                    off_w += item_weight(npt, tt, L);
                 }
             } else {
                 it.nprev = pt;
                 int slot = 0;
+                int off_i = off_g;
                 for (int tt = 0; tt < nq; ++tt) {
                     int e = (tt + 1) * T < L ? (tt + 1) * T : L;
                     int nself = ceil_div(e, BR_BN);
@@ -254,11 +254,19 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     }
     __syncthreads();
     if (tid == 0) {
-#pragma unroll
-        for (int g = 0; g < BR_NQUEUES; ++g) {
-            hdr[BR_PH_QCOUNT + g] = qbase[g];
-            hdr[BR_PH_QOFF + g] = qoff[g];
+        // a queue that received no item starts where the next one starts
+        const int end = n_glob_total + n_x_total;
+        int nxt = end;
+        for (int g = 7; g >= 0; --g) {
+            int f = s_qfirst[g];
+            if (f == 0x7fffffff) f = nxt;
+            hdr[BR_PH_QOFF + g] = f;
+            hdr[BR_PH_QCOUNT + g] = nxt - f;
+            nxt = f;
         }
+        hdr[BR_PH_QOFF + BR_GLOBAL_QUEUE] = 0;
+        hdr[BR_PH_QCOUNT + BR_GLOBAL_QUEUE] = n_glob_total;
+        const int base_items = end;
         hdr[BR_PH_NITEMS] = base_items;
         hdr[BR_PH_NCOMB] = base_comb;
         hdr[BR_PH_NONCONTIG] = s_bad;

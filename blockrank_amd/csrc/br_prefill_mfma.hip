@@ -86,6 +86,12 @@ __device__ inline int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 
 // is requested, and at the end of the item it is published through LDS.  Each step consumes a value
 // whose load was issued a whole tile earlier, so the chain ticket -> item costs the item's critical
 // path nothing (an item with a single tile finishes the chain at its end, waiting as needed).
+//
+// A workgroup draws from the global queue, then from the queue of its XCD (by workgroup index: the
+// hardware deals workgroups round robin to the XCDs), and is done when both are dry.  It does not look into the other XCDs' queues: the plan cuts the work into eight runs of
+// equal estimated size, and polling other queues' counters at the end of the kernel (with atomics
+// or with loads) was measured to stretch the memory waits of every workgroup still working from
+// 0.1 to 5-15 us.
 struct BrDescMail {      // layout of one LDS mailbox
     int word[BR_ITEM_INTS];
     int hg;
@@ -96,62 +102,104 @@ struct BrDescMail {      // layout of one LDS mailbox
 struct BrPrefetch {
     int* hdr;
     const BrPlanView* pv;
-    int NHG, xcc, lane;
-    int qk;        // step in the queue order (global, this XCD's, the others)
-    int counts;    // lane j: work units in queue j
+    int NHG, lane;
+    int xq, ng;    // this workgroup serves the XCD queues xq, xq + ng, ... (ng = 8 unless the grid is smaller)
+    int qk, qend;  // step in the queue order: 0 global queue, 1.. own queues, qend done
+    int counts;    // lane j: tickets of queue j
     int qoffs;     // lane j: index of queue j's first item
+    int scounts;   // lane j: tickets of queue j handed out statically (one per workgroup, see init)
     int t_next;    // ticket drawn from the queue at step qk (lane 0), or -1
-    int stage;     // 0 ticket drawn, 2 item requested, 9 queue ran dry
+    int stage;     // 0 ticket drawn, 2 item requested, 9 nothing in flight
     int word, hg;
 
+    // The first ticket of every workgroup is fixed by its index, with no atomic (512 workgroups
+    // drawing from one counter at the same moment queue up for microseconds): workgroups 0..SG-1
+    // take the global queue's tickets 0..SG-1; the others take, in index order, the first tickets of
+    // the queue blockIdx & 7 (workgroups are dealt round robin to the XCDs, so this is normally the
+    // queue of the XCD they run on; if it is not, only locality is lost).  The counters therefore
+    // count the tickets drawn after the static ones.
     __device__ void init(int* hdr_, const BrPlanView* pv_, int NHG_, int lane_) {
         hdr = hdr_; pv = pv_; NHG = NHG_; lane = lane_;
-        xcc = br_xcc_id();
-        qk = 0;
         counts = lane < BR_NQUEUES ? hdr[BR_PH_QCOUNT + lane] * NHG : 0;
         qoffs = lane < BR_NQUEUES ? hdr[BR_PH_QOFF + lane] : 0;
+        const int grid = gridDim.x, me = blockIdx.x;
+        // Queue ownership goes by workgroup index, not by the XCD id the hardware reports: every queue
+        // then has its workgroups whatever the placement is, so all work is done in any case.
+        ng = grid < 8 ? grid : 8;
+        xq = me % ng;
+        qend = 1 + (8 - xq + ng - 1) / ng;
+        const int cg = __builtin_amdgcn_readlane(counts, BR_GLOBAL_QUEUE);
+        const int SG = grid < 8 ? 0 : (cg < grid ? cg : grid);      // (no static tickets on a tiny grid)
+        const int first = SG + ((lane - SG) & 7);                   // lane j < 8: first workgroup of queue j
+        const int nwg = first < grid ? (grid - 1 - first) / 8 + 1 : 0;
+        scounts = lane < 8 ? (nwg < counts ? nwg : counts) : (lane == BR_GLOBAL_QUEUE ? SG : 0);
+        if (grid < 8) scounts = 0;
+        qk = SG == cg ? 1 : 0;      // every global ticket handed out already: start at the XCD's own queue
         t_next = -1;
         stage = 9;
         word = hg = 0;
+        int q = -1, t = 0;
+        if (me < SG) {
+            q = BR_GLOBAL_QUEUE;
+            t = me;
+        } else if (grid >= 8) {
+            const int x = me & 7;
+            const int r = (me - __builtin_amdgcn_readlane(first, x)) >> 3;
+            if (r < __builtin_amdgcn_readlane(scounts, x)) {
+                q = x;
+                t = r;
+            }
+        }
+        if (q >= 0) request(q, t);
+    }
+    __device__ int queue_now() const { return qk == 0 ? BR_GLOBAL_QUEUE : xq + (qk - 1) * ng; }
+    __device__ void request(int q, int t) {   // ask for the item that ticket t of queue q names
+        const int li = t / NHG;
+        hg = t - li * NHG;
+        const int idx = __builtin_amdgcn_readlane(qoffs, q) + li;
+        word = reinterpret_cast<const int*>(pv->items + idx)[lane & (BR_ITEM_INTS - 1)];
+        stage = 2;
     }
     __device__ void draw() {   // at the start of an item
         t_next = -1;
         stage = 9;
-        if (qk < BR_NQUEUES) {
-            if (lane == 0) t_next = atomicAdd(&hdr[BR_PH_QTICKET + br_queue_at(qk, xcc)], 1);
+        if (qk < qend) {
+            if (lane == 0) t_next = atomicAdd(&hdr[BR_PH_QTICKET + queue_now()], 1);
             stage = 0;
         }
     }
     __device__ void step() {   // once per key tile, after the tile's arithmetic
         if (stage == 0) {
-            const int q = br_queue_at(qk, xcc);
-            const int t = __builtin_amdgcn_readfirstlane(t_next);
+            const int q = queue_now();
+            const int t = __builtin_amdgcn_readfirstlane(t_next) + __builtin_amdgcn_readlane(scounts, q);
             if (t < __builtin_amdgcn_readlane(counts, q)) {
-                const int li = t / NHG;
-                hg = t - li * NHG;
-                const int idx = __builtin_amdgcn_readlane(qoffs, q) + li;
-                word = reinterpret_cast<const int*>(pv->items + idx)[lane & (BR_ITEM_INTS - 1)];
-                stage = 2;
+                request(q, t);
             } else {
                 stage = 9;
+                ++qk;          // that queue is dry for good
             }
         }
     }
-    __device__ void publish(BrDescMail* mail) {   // at the end of an item
-        if (stage == 0) step();
-        if (stage == 9) {
-            // the queue ran dry (or nothing was drawn): look through the remaining queues now
-            int qt = -1;
-            if (lane == 0) qt = br_take_ticket(hdr, NHG, xcc, &qk, t_next);
-            qt = __builtin_amdgcn_readfirstlane(qt);
-            qk = __builtin_amdgcn_readfirstlane(qk);
-            if (qt < 0) {
-                if (lane == 0) mail->valid = 0;
-                return;
+    // Nothing in flight: draw now, from the global queue and then the own one.
+    __device__ bool find_work() {
+        while (qk < qend) {
+            const int q = queue_now();
+            int t = 0;
+            if (lane == 0) t = atomicAdd(&hdr[BR_PH_QTICKET + q], 1);
+            t = __builtin_amdgcn_readfirstlane(t) + __builtin_amdgcn_readlane(scounts, q);
+            if (t < __builtin_amdgcn_readlane(counts, q)) {
+                request(q, t);
+                return true;
             }
-            int item;
-            br_decode_ticket(*pv, qt, NHG, item, hg);
-            word = reinterpret_cast<const int*>(pv->items + item)[lane & (BR_ITEM_INTS - 1)];
+            ++qk;
+        }
+        return false;
+    }
+    __device__ void publish(BrDescMail* mail) {   // at the end of an item (and once before the first)
+        if (stage == 0) step();
+        if (stage == 9 && !find_work()) {
+            if (lane == 0) mail->valid = 0;
+            return;
         }
         if (lane < BR_ITEM_INTS) mail->word[lane] = word;
         if (lane == 0) {
