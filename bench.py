@@ -1,13 +1,18 @@
 #!/usr/bin/env python3
 """Benchmark of the BlockRank attention + per-document score path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg4|cfg5shape|cfg1] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5shape|cfg1] [--no-cpu-baseline]
 
 A step is one pass of the hot path over one batch already resident in HBM: the attention hook
 (block-sparse prefill attention of one layer, query/key/value as a Mistral layer hands them over)
 followed by the fused per-document score extraction.  The request plan (block table + work items) is
 built once per forward pass by the mask hook and shared by every layer, so it is built outside the
 timed region and its cost is reported separately (``plan_build_ms``).
+
+``--workload cfg3`` is the end-to-end case instead (BASELINE configs[2]): a random-initialised
+Mistral-7B-shaped decoder run by the layer-truncated ranking driver (layers 0..19 in full, of layer 20
+only what the scores need), B=8; its line reports requests/s of the whole forward and, from HIP events
+around each layer's attention kernel, that kernel's roofline fraction at this layout.
 
 Prints ONE JSON line: requests/s for the batch, plus
   roofline      the main attention kernel against the bf16 MFMA peak (FLOPs of unmasked
@@ -97,11 +102,92 @@ def cpu_baseline(layout, q, k, v, scale, dtype, budget_s=12.0):
                 ms_per_request=med * 1e3)
 
 
+def bench_model(args):
+    """cfg3: the truncated ranking forward of a Mistral-7B-shaped model with random weights."""
+    import blockrank_amd as br
+    from blockrank_amd import profiling, synthetic
+    from transformers import MistralConfig, MistralModel
+    dev = torch.device("cuda:0")
+    layer_idx = 20
+    cfg = MistralConfig(vocab_size=32768, hidden_size=4096, intermediate_size=14336, num_hidden_layers=layer_idx + 1,
+                        num_attention_heads=32, num_key_value_heads=8, head_dim=128, rope_theta=1e6, sliding_window=None,
+                        max_position_embeddings=32768)
+    br.register_triton_blockrank_attention()
+    torch.manual_seed(0)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            model = MistralModel(cfg)          # only the layers the driver runs are built: 0 .. layer_idx
+    finally:
+        torch.set_default_dtype(old)
+    model.eval()
+    model.set_attn_implementation("triton_blockrank")
+    layout = synthetic.random_layout(8, 64, 20, 96, 224, 32, seed=0)
+    B, S = layout.B, layout.S
+    ids = torch.randint(0, cfg.vocab_size, (B, S), generator=torch.Generator().manual_seed(1)).to(dev)
+    pos = layout.position_ids.to(dev)
+    valid = layout.valid.to(dev)
+    R = min(16, layout.H)
+    rows = torch.tensor([[R - 2, R - 1]] * B, dtype=torch.int32, device=dev)
+    ranker = br.TruncatedRanker(model, layer_idx)
+    steps = args.steps if args.steps is not None else 10
+    warmup = args.warmup if args.warmup is not None else 2
+    for _ in range(warmup):
+        scores = ranker(ids, valid, pos, rows=rows)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        scores = ranker(ids, valid, pos, rows=rows)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+    assert torch.isfinite(scores).all()
+    # the attention kernel of every layer of one more forward, from HIP events around it
+    pairs = []
+
+    class _Events:
+        def __iter__(self):
+            pairs.append(profiling.EventPair())
+            return iter(pairs[-1].handles)
+
+    ranker(ids, valid, pos, rows=rows, kernel_events=_Events())
+    torch.cuda.synchronize()
+    kern_ms = [p.elapsed_ms() for p in pairs]
+    kern_avg_ms = sum(kern_ms) / len(kern_ms)
+    pairs_n = layout.unmasked_pairs()
+    flops = 4.0 * 128 * pairs_n * 32
+    alg_bytes = float(layout.valid_tokens) * 128 * 2 * (2 * 32 + 2 * 8)
+    tflops = flops / (kern_avg_ms * 1e-3) / 1e12
+    gbs = alg_bytes / (kern_avg_ms * 1e-3) / 1e9
+    dense_flops = 2.0 * 218103808 * layout.valid_tokens * layer_idx      # the projections and MLPs of layers 0..19 (real tokens)
+    res = {
+        "metric": "ranking requests/sec (Mistral-7B-shaped decoder, layers 0-20, layer-truncated forward, 20 docs)",
+        "value": B / (ms_per_step * 1e-3), "unit": "requests/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "Mistral-7B-shaped decoder (random init), B=8, 64-token prefix + 20 docs U[96,224] + 32-token query, "
+                               "layers 0..19 in full and the score part of layer 20, bf16",
+                   "name": "cfg3", "batch": B, "blocks": layout.M, "block_len": layout.H, "valid_tokens": layout.valid_tokens,
+                   "padded_tokens": B * S, "unmasked_pairs": pairs_n, "launch": "eager"},
+        "prefill_tok_per_s": layout.valid_tokens / (ms_per_step * 1e-3),
+        "attention_ms_per_step": sum(kern_ms),
+        "attention_share": sum(kern_ms) / ms_per_step,
+        "dense_tflops": dense_flops / (ms_per_step * 1e-3) / 1e12,
+        "kernel_us": {"prefill_avg": kern_avg_ms * 1e3, "prefill_min": min(kern_ms) * 1e3, "prefill_max": max(kern_ms) * 1e3,
+                      "launches": len(kern_ms)},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tflops / PEAK_BF16_TFLOPS,
+                     "traffic": None, "kernel": "br_prefill_mfma_kernel", "flops_per_launch": flops},
+        "roofline_hbm": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                         "bytes_per_launch": alg_bytes},
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
@@ -114,6 +200,11 @@ def main():
                  "(run with --gpus 1)")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+
+    if args.workload == "cfg3":
+        return bench_model(args)
+    args.steps = 200 if args.steps is None else args.steps
+    args.warmup = 20 if args.warmup is None else args.warmup
 
     import blockrank_amd as br
     from blockrank_amd import profiling, synthetic

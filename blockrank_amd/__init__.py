@@ -6,6 +6,7 @@ src/blockrank/__init__.py:19-33):
     register_blockrank_attention, register_triton_blockrank_attention   attention-interface hooks
     compute_auxiliary_attention_loss                                    per-document scores
 
+``TruncatedRanker`` (the evaluation script's layer-truncated forward, scripts/eval_attn.py:102-151),
 plus the functional entry points ``blockrank_attention``, ``doc_scores``, ``last_block_logits`` and
 the ``BlockMask`` / ``LastBlockScores`` objects the hooks exchange.  Everything computes in
 hand-written HIP kernels (libblockrank_hip.so); there is no fallback implementation.
@@ -23,6 +24,7 @@ from .attention import (
     register_triton_blockrank_attention,
 )
 from .losses import compute_auxiliary_attention_loss, rank_documents
+from .ranker import TruncatedRanker
 
 __all__ = [
     "BlockMask",
@@ -37,5 +39,6 @@ __all__ = [
     "register_triton_blockrank_attention",
     "compute_auxiliary_attention_loss",
     "rank_documents",
+    "TruncatedRanker",
 ]
 __version__ = "0.1.0"

@@ -321,15 +321,17 @@ class LastBlockScores:
                                return_probs=return_probs)
 
 
-def _score_args(query, key, block_mask, rows):
+def _score_args(query, key, block_mask, rows, query_block_only=False):
     if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
         block_mask = BlockMask(block_mask, query.dtype)
     bm = _as_block_mask(block_mask)
     if not query.is_cuda:
         raise RuntimeError("blockrank_amd runs on a GPU only (got CPU tensors); it has no CPU fallback")
-    B, Nq, S, D = query.shape
-    Nkv = key.shape[1]
+    B, Nq, Sq, D = query.shape
+    Nkv, S = key.shape[1], key.shape[2]
     assert bm.M * bm.H == S, "attention mask does not match the sequence length"
+    assert Sq == (bm.H if query_block_only else S), "query must cover the query block only" if query_block_only else \
+        "query and key must cover the same tokens"
     if query.dtype not in _DTYPE_CODE:
         raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
     assert rows.dim() == 2 and rows.shape[0] == B, "rows must be (B, R)"
@@ -341,15 +343,18 @@ def _score_args(query, key, block_mask, rows):
 
 
 def doc_scores(query, key, block_mask, rows, scaling: float, temperature: float = 0.05, head_reduce: str = "mean",
-               row_reduce: str = "mean", return_probs: bool = False):
+               row_reduce: str = "mean", return_probs: bool = False, query_block_only: bool = False):
     """Fused per-document relevance: for every (head, chosen query-block row) a softmax of
     scaling*q.k over all real document tokens, summed per document, reduced over heads and rows and
     divided by the temperature.  Equals compute_auxiliary_attention_loss(s_last, ..., answer_ids=None,
     return_logits=True) (src/blockrank/losses.py:37-78) with rows = the bracket row and the one before.
 
     rows: (B, R) positions inside the query block (0..H-1), R <= 16.  Returns (B, M-2) fp32, and the
-    (B, Nq, R, M-2) per-head probabilities too if return_probs."""
-    bm, q, k, rows, (B, Nq, Nkv, S, D) = _score_args(query, key, block_mask, rows)
+    (B, Nq, R, M-2) per-head probabilities too if return_probs.
+
+    query_block_only: ``query`` holds the query block's H tokens only, (B, Nq, H, D) - for callers that
+    never project the other tokens' queries (the kernels read no other query rows)."""
+    bm, q, k, rows, (B, Nq, Nkv, S, D) = _score_args(query, key, block_mask, rows, query_block_only)
     R = rows.shape[1]
     assert bm.M >= 3, "per-document scores need at least one document block"
     assert head_reduce in ("mean", "sum") and row_reduce in ("mean", "sum")
@@ -366,8 +371,10 @@ def doc_scores(query, key, block_mask, rows, scaling: float, temperature: float 
         probs = torch.empty((B, Nq, R, bm.M - 2), dtype=torch.float32, device=dev) if return_probs else None
         ws_bytes = lib.br_doc_scores_workspace_bytes(B, Nq, bm.M, R)
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        # the kernels address query rows as token (M-1)*H + position: shift the base accordingly
+        q_ptr = q.data_ptr() - ((bm.M - 1) * bm.H * q.stride(2) * q.element_size() if query_block_only else 0)
         _lib.check(lib.br_doc_scores(
-            q.data_ptr(), k.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, B, Nq, Nkv, bm.M, bm.H, D,
+            q_ptr, k.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, B, Nq, Nkv, bm.M, bm.H, D,
             _lib.strides3(q), _lib.strides3(k), float(scaling), float(out_scale), _DTYPE_CODE[query.dtype],
             scores.data_ptr(), probs.data_ptr() if probs is not None else None, ws.data_ptr(), ws_bytes, _stream_ptr(dev)))
     return (scores, probs) if return_probs else scores

@@ -124,7 +124,9 @@ size_t br_doc_scores_workspace_bytes(int B, int Nq, int M, int R);
  *   scores: (B, M-2) fp32 = out_scale * sum over heads and rows of the document's probability mass
  *   under a softmax of scale*q.k over all real document tokens.  The reference's mean over heads and
  *   rows divided by the temperature is out_scale = 1 / (Nq * R * temperature).
- *   probs: optional (B, Nq, R, M-2) fp32 per-head, per-row document probabilities, or NULL. */
+ *   probs: optional (B, Nq, R, M-2) fp32 per-head, per-row document probabilities, or NULL.
+ *   Of q only the rows named by `rows` are read (tokens (M-1)*H + rows[b][r]), so a caller that has
+ *   projected the query block alone may pass a base pointer shifted accordingly. */
 int br_doc_scores(const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B, int Nq,
                   int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, float scale,
                   float out_scale, int dtype, float* scores, float* probs, void* workspace, size_t workspace_bytes,

@@ -76,3 +76,29 @@ def test_every_reference_impl_name_is_registered():
                  "sdpa_compiled_blockrank", "triton_blockrank", "triton_blockrank_compiled"]:
         assert AttentionInterface()[name] is br.blockrank_attention_forward
         assert AttentionMaskInterface()[name] is br.blockrank_attention_mask
+
+
+@pytest.mark.parametrize("kind,dtype", [("mistral", torch.float32), ("mistral", torch.bfloat16), ("qwen2", torch.bfloat16)])
+def test_truncated_ranker_matches_full_forward(kind, dtype):
+    """The layer-truncated driver (scripts/eval_attn.py:102-151 counterpart) returns the scores of the full
+    forward + compute_auxiliary_attention_loss, for the scoring layer in the middle and at the start."""
+    br.register_triton_blockrank_attention()
+    model = build(kind, dtype)
+    model.set_attn_implementation("triton_blockrank")
+    lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
+    lay.labels[:] = -100
+    lay.labels[:, -2:] = 7                                   # "[" is the second to last token
+    B, S = lay.B, lay.S
+    ids = torch.randint(0, 512, (B, S), generator=torch.Generator().manual_seed(3)).to(DEV)
+    pos = lay.position_ids.to(DEV)
+    valid = lay.valid.to(DEV)
+    for layer_idx in (1, 0, 2):
+        with torch.no_grad():
+            full = model(input_ids=ids, position_ids=pos, attention_mask=valid, output_attentions=True,
+                         layers_to_return_scores=[layer_idx], use_cache=False)
+        want = br.compute_auxiliary_attention_loss(full.attentions[0], lay.labels.to(DEV), valid, answer_ids=None, return_logits=True)
+        ranker = br.TruncatedRanker(model, layer_idx)
+        got = ranker(ids, valid, pos, labels=lay.labels.to(DEV))
+        assert got.shape == (B, lay.M - 2)
+        torch.testing.assert_close(got, want, rtol=2e-3 if dtype == torch.bfloat16 else 1e-4, atol=1e-5)
+        assert torch.equal(ranker.rank(ids, valid, pos, labels=lay.labels.to(DEV), k=3), br.rank_documents(want, 3))
