@@ -25,6 +25,7 @@ from .attention import (
 )
 from .losses import compute_auxiliary_attention_loss, rank_documents
 from .ranker import TruncatedRanker
+from .collate import block_icr_collate_packed, pack_padded_batch
 
 __all__ = [
     "BlockMask",
@@ -40,5 +41,7 @@ __all__ = [
     "compute_auxiliary_attention_loss",
     "rank_documents",
     "TruncatedRanker",
+    "block_icr_collate_packed",
+    "pack_padded_batch",
 ]
 __version__ = "0.1.0"

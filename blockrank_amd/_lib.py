@@ -28,6 +28,7 @@ SIGNATURES = {
     "br_plan_ints": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "br_plan_build": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "br_plan_build_from_lengths": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "br_plan_build_packed": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "br_prefill_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "br_prefill_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t, c_void_p]),
@@ -90,7 +91,8 @@ def check(rc: int) -> None:
     raise RuntimeError(f"libblockrank_hip error {rc}: {msg}")
 
 
-def strides3(t) -> ctypes.Array:
-    """Element strides (batch, head, token) of a logical (B, heads, S, D) tensor."""
+def strides3(t, packed: bool = False) -> ctypes.Array:
+    """Element strides (batch, head, token) of a logical (B, heads, S, D) tensor; a packed layout has
+    one token axis for the whole batch, i.e. batch stride 0."""
     s = t.stride()
-    return _I64x3(s[0], s[1], s[2])
+    return _I64x3(0 if packed else s[0], s[1], s[2])

@@ -59,9 +59,50 @@ class BlockMask:
         if not valid.is_cuda:
             raise RuntimeError("blockrank_amd runs on a GPU only: the block attention mask must be a CUDA/HIP tensor")
         self.valid = valid.bool().contiguous()
+        self.lengths = None
+        self.packed = False
+        self.left_padded = True
+        self.total_tokens = None
         self.dtype = dtype
         self.B, self.M, self.H = valid.shape
         self._plans: dict[tuple[int, int], torch.Tensor] = {}
+
+    @classmethod
+    def from_lengths(cls, lengths: torch.Tensor, H: Optional[int] = None, packed: bool = False, left_padded: bool = True,
+                     dtype: torch.dtype = torch.float32) -> "BlockMask":
+        """From per-block real-token counts (B, M) instead of a padded mask.
+
+        packed=False describes the reference's padded layout (every block in H slots, its tokens at the
+        left or right end of them).  packed=True describes tensors with no padded slots at all: the
+        tokens of all blocks of all sequences follow each other on one token axis, q/k/v are
+        (1, heads, T, D) with T = lengths.sum(); H is then only an upper bound of the block lengths
+        (default: the maximum rounded up to 16) and the coordinate system of score rows."""
+        assert lengths.dim() == 2, "lengths must be (B, M)"
+        if not lengths.is_cuda:
+            raise RuntimeError("blockrank_amd runs on a GPU only: the block lengths must be a CUDA/HIP tensor")
+        self = cls.__new__(cls)
+        self.valid = None
+        self.lengths = lengths.to(torch.int32).contiguous()
+        self.packed = bool(packed)
+        self.left_padded = bool(left_padded)
+        host = None
+        if H is None or packed:
+            host = lengths.cpu()
+        if H is None:
+            H = (int(host.max()) + 15) // 16 * 16
+        self.total_tokens = int(host.sum()) if packed else None
+        self.dtype = dtype
+        self.B, self.M = lengths.shape
+        self.H = int(H)
+        self._plans = {}
+        return self
+
+    def _valid_mask(self) -> torch.Tensor:
+        if self.valid is None:
+            j = torch.arange(self.H, device=self.lengths.device)[None, None, :]
+            ln = self.lengths[:, :, None]
+            self.valid = (j >= self.H - ln) if self.left_padded else (j < ln)
+        return self.valid
 
     # -- what the reference's 5-D tensor would answer ------------------------------------------
     @property
@@ -70,7 +111,7 @@ class BlockMask:
 
     @property
     def device(self):
-        return self.valid.device
+        return self.valid.device if self.valid is not None else self.lengths.device
 
     def dim(self) -> int:
         return 5
@@ -86,7 +127,10 @@ class BlockMask:
         0.7 * finfo(dtype).min (blockrank_std_attention.py:297-307)."""
         dtype = dtype or self.dtype
         B, M, H = self.B, self.M, self.H
-        keep = self.valid.view(B, 1, M, 1, H) & torch.tril(torch.ones(H, H, dtype=torch.bool, device=self.valid.device))
+        if self.packed:
+            raise NotImplementedError("a packed layout has no padded (B, 1, M, H, H) mask tensor")
+        valid = self._valid_mask()
+        keep = valid.view(B, 1, M, 1, H) & torch.tril(torch.ones(H, H, dtype=torch.bool, device=valid.device))
         neg = 0.7 * torch.finfo(dtype).min
         return torch.where(keep, torch.zeros((), dtype=dtype, device=keep.device), torch.full((), neg, dtype=dtype, device=keep.device))
 
@@ -105,10 +149,18 @@ class BlockMask:
             lib = _lib.load()
             n = lib.br_plan_ints(self.B, self.M, self.H, Nq, Nkv)
             assert n > 0, f"unsupported head layout: {Nq} query heads, {Nkv} kv heads"
-            with torch.cuda.device(self.valid.device):
-                plan = torch.empty(n, dtype=torch.int32, device=self.valid.device)
-                _lib.check(lib.br_plan_build(self.valid.data_ptr(), self.B, self.M, self.H, Nq, Nkv, plan.data_ptr(), n,
-                                             _stream_ptr(self.valid.device)))
+            dev = self.device
+            with torch.cuda.device(dev):
+                plan = torch.empty(n, dtype=torch.int32, device=dev)
+                if self.lengths is None:
+                    _lib.check(lib.br_plan_build(self.valid.data_ptr(), self.B, self.M, self.H, Nq, Nkv, plan.data_ptr(), n,
+                                                 _stream_ptr(dev)))
+                elif self.packed:
+                    _lib.check(lib.br_plan_build_packed(self.lengths.data_ptr(), self.B, self.M, self.H, Nq, Nkv,
+                                                        plan.data_ptr(), n, _stream_ptr(dev)))
+                else:
+                    _lib.check(lib.br_plan_build_from_lengths(self.lengths.data_ptr(), int(self.left_padded), self.B, self.M,
+                                                              self.H, Nq, Nkv, plan.data_ptr(), n, _stream_ptr(dev)))
             if _env_flag("BLOCKRANK_AMD_DEBUG"):
                 # same role as the reference's _DEBUG left-padding check (blockrank_std_attention.py:146-148)
                 assert int(plan[4].item()) == 0, "Attention mask is not one contiguous span of real tokens per block"
@@ -117,7 +169,7 @@ class BlockMask:
 
     def block_lengths(self) -> torch.Tensor:
         """(B, M) int32 number of real tokens per block."""
-        return self.valid.sum(-1, dtype=torch.int32)
+        return self.lengths if self.lengths is not None else self.valid.sum(-1, dtype=torch.int32)
 
 
 def blockrank_attention_mask(
@@ -194,12 +246,15 @@ def blockrank_attention(
     bm = _as_block_mask(block_mask)
     if not query.is_cuda:
         raise RuntimeError("blockrank_amd runs on a GPU only (got CPU tensors); it has no CPU fallback")
-    B, Nq, S, D = query.shape
+    Bt, Nq, S, D = query.shape
     Nkv = key.shape[1]
-    M, H = bm.M, bm.H
-    assert H == S // M and M * H == S, f"Block size H={H} does not match MH // M = {S // M}"
-    assert key.shape == (B, Nkv, S, D) and value.shape == (B, Nkv, S, D), "key/value must be (B, Nkv, S, D)"
-    assert bm.B == B, "attention mask batch size does not match query"
+    M, H, B, packed = bm.M, bm.H, bm.B, bm.packed
+    if packed:
+        assert Bt == 1 and S == bm.total_tokens, "a packed layout takes (1, heads, T, D) tensors with T = sum of block lengths"
+    else:
+        assert H == S // M and M * H == S, f"Block size H={H} does not match MH // M = {S // M}"
+        assert Bt == B, "attention mask batch size does not match query"
+    assert key.shape == (Bt, Nkv, S, D) and value.shape == (Bt, Nkv, S, D), "key/value must be (B, Nkv, S, D)"
     if query.dtype not in _DTYPE_CODE:
         raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
     assert key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value must share a dtype"
@@ -214,24 +269,24 @@ def blockrank_attention(
     dev = query.device
     with torch.cuda.device(dev):
         plan = bm.plan(Nq, Nkv)
-        out = torch.empty((B, S, Nq, D), dtype=query.dtype, device=dev)
+        out = torch.empty((Bt, S, Nq, D), dtype=query.dtype, device=dev)
         ws_bytes = lib.br_prefill_workspace_bytes(B, Nq, Nkv, D)
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-        out_strides = _lib._I64x3(S * Nq * D, D, Nq * D)
+        out_strides = _lib._I64x3(0 if packed else S * Nq * D, D, Nq * D)
         ev0, ev1 = kernel_events if kernel_events is not None else (None, None)
         if score_rows > 0:
             sp_bytes = lib.br_score_partials_bytes(B, Nq, M, H, score_rows)
             part = torch.empty(max(sp_bytes // 4, 4), dtype=torch.float32, device=dev)
             _lib.check(lib.br_prefill_fwd_scores(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
-                _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), out_strides, float(scaling),
+                _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed), out_strides, float(scaling),
                 _DTYPE_CODE[query.dtype], ws.data_ptr(), ws_bytes, score_rows, part.data_ptr(), sp_bytes,
                 _stream_ptr(dev), ev0, ev1))
             return out, part
         _lib.check(lib.br_prefill_fwd_events(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
-            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), out_strides, float(scaling), _DTYPE_CODE[query.dtype],
-            ws.data_ptr(), ws_bytes, _stream_ptr(dev), ev0, ev1))
+            _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed), out_strides, float(scaling),
+            _DTYPE_CODE[query.dtype], ws.data_ptr(), ws_bytes, _stream_ptr(dev), ev0, ev1))
     return out
 
 
@@ -281,8 +336,8 @@ class LastBlockScores:
         self.query, self.key, self.block_mask = query, key, block_mask
         self.scaling, self.R, self.scaled = float(scaling), int(num_rows), scaled
         self.partials = partials if scaled else None    # per-tile (max, sum) pairs left by the attention kernel
-        B, Nq, S, D = query.shape
-        self.shape = torch.Size((B, Nq, self.R, S))
+        _, Nq, _, D = query.shape
+        self.shape = torch.Size((block_mask.B, Nq, self.R, block_mask.M * block_mask.H))
         self.device, self.dtype = query.device, query.dtype
 
     def dim(self) -> int:
@@ -327,11 +382,16 @@ def _score_args(query, key, block_mask, rows, query_block_only=False):
     bm = _as_block_mask(block_mask)
     if not query.is_cuda:
         raise RuntimeError("blockrank_amd runs on a GPU only (got CPU tensors); it has no CPU fallback")
-    B, Nq, Sq, D = query.shape
+    _, Nq, Sq, D = query.shape
     Nkv, S = key.shape[1], key.shape[2]
-    assert bm.M * bm.H == S, "attention mask does not match the sequence length"
-    assert Sq == (bm.H if query_block_only else S), "query must cover the query block only" if query_block_only else \
-        "query and key must cover the same tokens"
+    B = bm.B
+    if bm.packed:
+        assert key.shape[0] == 1 and S == bm.total_tokens, "a packed layout takes (1, heads, T, D) tensors"
+        assert not query_block_only and Sq == S, "a packed layout takes the query tensor over all T tokens"
+    else:
+        assert bm.M * bm.H == S, "attention mask does not match the sequence length"
+        assert Sq == (bm.H if query_block_only else S), "query must cover the query block only" if query_block_only else \
+            "query and key must cover the same tokens"
     if query.dtype not in _DTYPE_CODE:
         raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
     assert rows.dim() == 2 and rows.shape[0] == B, "rows must be (B, R)"
@@ -375,7 +435,7 @@ def doc_scores(query, key, block_mask, rows, scaling: float, temperature: float 
         q_ptr = q.data_ptr() - ((bm.M - 1) * bm.H * q.stride(2) * q.element_size() if query_block_only else 0)
         _lib.check(lib.br_doc_scores(
             q_ptr, k.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, B, Nq, Nkv, bm.M, bm.H, D,
-            _lib.strides3(q), _lib.strides3(k), float(scaling), float(out_scale), _DTYPE_CODE[query.dtype],
+            _lib.strides3(q, bm.packed), _lib.strides3(k, bm.packed), float(scaling), float(out_scale), _DTYPE_CODE[query.dtype],
             scores.data_ptr(), probs.data_ptr() if probs is not None else None, ws.data_ptr(), ws_bytes, _stream_ptr(dev)))
     return (scores, probs) if return_probs else scores
 
@@ -391,11 +451,12 @@ def last_block_logits(query, key, block_mask, rows, scaling: float, neg: Optiona
     dev = query.device
     with torch.cuda.device(dev):
         plan = bm.plan(Nq, Nkv)
-        out = torch.empty((B, Nq, R, S), dtype=torch.float32, device=dev)
+        # (for a packed layout too the result is laid out over the M*H padded key slots, like the reference's)
+        out = torch.empty((B, Nq, R, bm.M * bm.H), dtype=torch.float32, device=dev)
         _lib.check(lib.br_last_block_logits(
             q.data_ptr(), k.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, B, Nq, Nkv, bm.M, bm.H, D,
-            _lib.strides3(q), _lib.strides3(k), float(scaling), float(neg), _DTYPE_CODE[query.dtype], out.data_ptr(),
-            _stream_ptr(dev)))
+            _lib.strides3(q, bm.packed), _lib.strides3(k, bm.packed), float(scaling), float(neg), _DTYPE_CODE[query.dtype],
+            out.data_ptr(), _stream_ptr(dev)))
     return out
 
 
@@ -425,7 +486,8 @@ def blockrank_attention_forward(
     assert attention_mask is not None, "BlockRank attention requires an attention mask"
     bm = _as_block_mask(attention_mask)
     B, Nq, S, D = query.shape
-    assert bm.H == S // bm.M, f"Block size H={bm.H} does not match MH // M = {S // bm.M}"
+    if not bm.packed:
+        assert bm.H == S // bm.M, f"Block size H={bm.H} does not match MH // M = {S // bm.M}"
     groups = getattr(module, "num_key_value_groups", None)
     if groups is not None:
         assert key.shape[1] * groups == Nq, "num_key_value_groups does not match the query/key head counts"

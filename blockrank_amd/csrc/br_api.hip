@@ -7,7 +7,7 @@
 #include "../../include/blockrank_hip.h"
 #include "br_common.h"
 
-void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int B, int M, int H, int T, int* plan,
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int* plan,
                     hipStream_t stream);
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                            hipEvent_t ev_start, hipEvent_t ev_stop);
@@ -126,7 +126,7 @@ size_t br_plan_ints(int B, int M, int H, int Nq, int Nkv) {
     return br_plan_total_ints(B, M, H, br_tokens_per_tile(g));
 }
 
-static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded, int B, int M, int H, int Nq, int Nkv,
+static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded, int packed, int B, int M, int H, int Nq, int Nkv,
                       int32_t* plan, size_t plan_ints, void* stream) {
     if (B <= 0 || M <= 0 || H <= 0) return fail(BR_ERR_ARG, "B, M and H must be positive (got %d, %d, %d)", B, M, H);
     BrGeom g;
@@ -139,19 +139,24 @@ static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded
     if (plan_ints < need) return fail(BR_ERR_SPACE, "plan buffer holds %zu ints, %zu needed", plan_ints, need);
     if ((long long)br_plan_max_items(B, M, H, T) * g.NHG >= (1 << 24))
         return fail(BR_ERR_ARG, "batch too large for one plan (B=%d, M=%d, H=%d)", B, M, H);
-    br_launch_plan(valid, lens, left_padded, B, M, H, T, plan, static_cast<hipStream_t>(stream));
+    br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, plan, static_cast<hipStream_t>(stream));
     return check_launch("plan launch");
 }
 
 int br_plan_build(const uint8_t* valid, int B, int M, int H, int Nq, int Nkv, int32_t* plan, size_t plan_ints, void* stream) {
     if (!valid) return fail(BR_ERR_ARG, "attention mask must be provided");
-    return plan_build(valid, nullptr, 1, B, M, H, Nq, Nkv, plan, plan_ints, stream);
+    return plan_build(valid, nullptr, 1, 0, B, M, H, Nq, Nkv, plan, plan_ints, stream);
 }
 
 int br_plan_build_from_lengths(const int32_t* lens, int left_padded, int B, int M, int H, int Nq, int Nkv, int32_t* plan,
                                size_t plan_ints, void* stream) {
     if (!lens) return fail(BR_ERR_ARG, "block lengths must be provided");
-    return plan_build(nullptr, lens, left_padded, B, M, H, Nq, Nkv, plan, plan_ints, stream);
+    return plan_build(nullptr, lens, left_padded, 0, B, M, H, Nq, Nkv, plan, plan_ints, stream);
+}
+
+int br_plan_build_packed(const int32_t* lens, int B, int M, int H, int Nq, int Nkv, int32_t* plan, size_t plan_ints, void* stream) {
+    if (!lens) return fail(BR_ERR_ARG, "block lengths must be provided");
+    return plan_build(nullptr, lens, 1, 1, B, M, H, Nq, Nkv, plan, plan_ints, stream);
 }
 
 size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {

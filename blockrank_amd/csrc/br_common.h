@@ -16,7 +16,7 @@
 #define BR_MIN_CHUNK 8        // a split of the query block's key walk covers at least this many tiles
 
 // Plan buffer (int32):
-//   [header BR_PLAN_HDR][start B*M][len B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
+//   [header BR_PLAN_HDR][start B*M][len B*M][tok B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
 //   [items 16*max_items][comb 4*max_comb]
 // Tile descriptors: for each sequence, the 64-key tiles of blocks 0..M-2 in order, as (token index of
 // the tile's first key, number of real keys); TPS = (M-1) * ceil(H/64) slots per sequence.
@@ -32,6 +32,7 @@
 enum BrPlanHeader {
     BR_PH_NITEMS = 0,     // number of work items (per head group)
     BR_PH_NCOMB = 1,      // number of combine entries (per head group)
+    BR_PH_PACKED = 2,     // 1: tokens are packed (no padded slots between blocks), see tok[] below
     BR_PH_NONCONTIG = 4,  // set to 1 if some block's real tokens are not one contiguous span
     BR_PH_MAX_ITEMS = 5,
     BR_PH_MAX_COMB = 6,
@@ -53,8 +54,10 @@ enum BrPlanHeader {
 struct BrItem {
     int b, m, t0, f_lo, nprev, ntiles, slot, pe;
     int len_m, start_m, len0, start0;
-    int pad[4];
+    int tok_m, tok0;      // index on the token axis of the first real token of block m / of block 0
+    int pad[2];
 };
+#define BR_ITEM_WORDS_USED 14
 #define BR_ITEM_INTS 16
 struct BrComb {
     int b, t0, slot0, nsplit;
@@ -62,8 +65,11 @@ struct BrComb {
 
 struct BrPlanView {
     const int* hdr;
-    const int* start;      // B*M
+    const int* start;      // B*M: position of the block's first real token inside its H slots
     const int* len;        // B*M
+    const int* tok;        // B*M: index of that token on the token axis of q/k/v/out.  Padded layout:
+                           // m*H + start (per sequence); packed layout: running sum of the lengths
+                           // over the whole batch (the batch stride of the tensors is then 0)
     const int2* tiles;     // B * TPS tile descriptors
     int tps;
     const BrItem* items;
@@ -72,7 +78,8 @@ struct BrPlanView {
 
 __host__ __device__ inline size_t br_plan_off_start() { return BR_PLAN_HDR; }
 __host__ __device__ inline size_t br_plan_off_len(int B, int M) { return BR_PLAN_HDR + (size_t)B * M; }
-__host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M; }
+__host__ __device__ inline size_t br_plan_off_tok(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M; }
+__host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLAN_HDR + 3 * (size_t)B * M; }
 __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
     int qt = (H + T - 1) / T;
     int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
@@ -80,7 +87,7 @@ __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
 }
 __host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }
 __host__ __device__ inline int br_plan_tps(int M, int H) { return (M > 1 ? M - 1 : 0) * ((H + BR_BN - 1) / BR_BN); }
-__host__ __device__ inline size_t br_plan_off_tbase(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M + (size_t)B; }
+__host__ __device__ inline size_t br_plan_off_tbase(int B, int M) { return BR_PLAN_HDR + 3 * (size_t)B * M + (size_t)B; }
 __host__ __device__ inline size_t br_plan_off_tiles(int B, int M) { return (br_plan_off_tbase(B, M) + (size_t)B * M + 1) & ~(size_t)1; }
 __host__ __device__ inline size_t br_plan_off_items(int B, int M, int H, int T) {
     size_t o = br_plan_off_tiles(B, M) + 2 * (size_t)B * br_plan_tps(M, H);
@@ -98,6 +105,7 @@ __device__ inline BrPlanView br_plan_view(const int* plan, int B, int M, int H, 
     v.hdr = plan;
     v.start = plan + br_plan_off_start();
     v.len = plan + br_plan_off_len(B, M);
+    v.tok = plan + br_plan_off_tok(B, M);
     v.tiles = reinterpret_cast<const int2*>(plan + br_plan_off_tiles(B, M));
     v.tps = br_plan_tps(M, H);
     v.items = reinterpret_cast<const BrItem*>(plan + br_plan_off_items(B, M, H, T));
@@ -174,7 +182,7 @@ struct BrWalk {
         f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
         nprev = it.nprev;
         self_end = self_end_;
-        own_tok0 = it.m * H + it.start_m;
+        own_tok0 = it.tok_m;
     }
     // returns 0: exhausted, 1: earlier-block tile *prev_index, 2: own tile filled into t
     __device__ int next(BrTile& t, int* prev_index) {
@@ -198,7 +206,7 @@ struct BrWalk {
 // Descriptor of earlier-block tile i of a document (the only earlier block is the prefix).
 __device__ inline void br_prefix_tile(const BrItem& it, int i, BrTile& t) {
     t.flat = i;
-    t.tok0 = it.start0 + i * BR_BN;
+    t.tok0 = it.tok0 + i * BR_BN;
     t.kt = i;
     t.nvalid = it.len0 - i * BR_BN < BR_BN ? it.len0 - i * BR_BN : BR_BN;
     t.self = 0;

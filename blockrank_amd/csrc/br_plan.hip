@@ -74,13 +74,14 @@ __device__ inline int splits_for(int ntiles, int ns_cap) {
     return ns > ns_cap ? ns_cap : ns;
 }
 
-__global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T) {
+__global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T, int packed) {
     __shared__ int sh[kPlanThreads / 64];
     __shared__ int s_bad;
     const int tid = threadIdx.x;
     int* hdr = plan;
     int* start = plan + br_plan_off_start();
     int* len = plan + br_plan_off_len(B, M);
+    int* tok = plan + br_plan_off_tok(B, M);
     int* prev_tiles = plan + br_plan_off_prev(B, M);
     int* tbase = plan + br_plan_off_tbase(B, M);
     int2* tiles = reinterpret_cast<int2*>(plan + br_plan_off_tiles(B, M));
@@ -101,6 +102,20 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         }
     }
     __syncthreads();
+    // where each block's first real token sits on the token axis
+    if (!packed) {
+        for (int p = tid; p < BM; p += kPlanThreads) tok[p] = (p % M) * H + start[p];
+    } else {
+        int base = 0;
+        for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
+            const int p = p0 + tid;
+            int tot;
+            const int ex = block_exclusive_scan(p < BM ? len[p] : 0, sh, &tot);
+            if (p < BM) tok[p] = base + ex;
+            base += tot;
+        }
+    }
+    __syncthreads();
     for (int b = tid; b < B; b += kPlanThreads) {
         int s = 0;
         for (int m = 0; m < M - 1; ++m) {
@@ -114,9 +129,9 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     for (int p = tid; p < BM; p += kPlanThreads) {
         const int b = p / M, m = p - b * M;
         if (m == M - 1) continue;
-        const int L = len[p], st = start[p];
+        const int L = len[p];
         for (int kt = 0; kt * BR_BN < L; ++kt)
-            tiles[(size_t)b * tps + tbase[p] + kt] = make_int2(m * H + st + kt * BR_BN, L - kt * BR_BN < BR_BN ? L - kt * BR_BN : BR_BN);
+            tiles[(size_t)b * tps + tbase[p] + kt] = make_int2(tok[p] + kt * BR_BN, L - kt * BR_BN < BR_BN ? L - kt * BR_BN : BR_BN);
     }
     __syncthreads();
 
@@ -214,7 +229,8 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             BrItem it;
             it.b = b; it.m = m; it.pe = pe;
             it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
-            it.pad[0] = it.pad[1] = it.pad[2] = it.pad[3] = 0;
+            it.tok_m = tok[b * M + m]; it.tok0 = tok[b * M];
+            it.pad[0] = it.pad[1] = 0;
             if (!is_last) {
                 it.nprev = npt;
                 for (int tt = 0; tt < nq; ++tt) {
@@ -269,6 +285,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         const int base_items = end;
         hdr[BR_PH_NITEMS] = base_items;
         hdr[BR_PH_NCOMB] = base_comb;
+        hdr[BR_PH_PACKED] = packed;
         hdr[BR_PH_NONCONTIG] = s_bad;
         hdr[BR_PH_MAX_ITEMS] = max_items;
         hdr[BR_PH_MAX_COMB] = br_plan_max_comb(B);
@@ -290,7 +307,7 @@ __global__ void br_block_table_from_len_kernel(const int* __restrict__ lens, int
 
 }  // namespace
 
-void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int B, int M, int H, int T, int* plan,
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int* plan,
                     hipStream_t stream) {
     int* start = plan + br_plan_off_start();
     int* len = plan + br_plan_off_len(B, M);
@@ -303,5 +320,5 @@ void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int 
         hipLaunchKernelGGL(br_block_table_from_len_kernel, dim3((BM + 255) / 256), dim3(256), 0, stream, lens, BM, H,
                            left_padded, start, len);
     }
-    hipLaunchKernelGGL(br_plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, plan, B, M, H, T);
+    hipLaunchKernelGGL(br_plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, plan, B, M, H, T, packed);
 }

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(NW * 64) void br_prefill_f32_kernel(BrPrefillParams
         const int row = it.t0 + sub * BR_RB + n;           // this lane pair's query row, valid-relative
         const bool row_ok = row < len_m;
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
-        const int qtok0 = m * p.H + it.start_m;
+        const int qtok0 = it.tok_m;
 
         float q[HD], o[HD];
         {
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void br_combine_f32_kernel(BrPrefillParams p, 
         const BrComb c = pv.comb[ci];
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int len_m = pv.len[c.b * p.M + m];
-        const int qtok0 = m * p.H + pv.start[c.b * p.M + m];
+        const int qtok0 = pv.tok[c.b * p.M + m];
         const int rows = NW * BR_RB;
         for (int idx = threadIdx.x; idx < rows * D; idx += blockDim.x) {
             const int r = idx / D, d = idx - r * D;
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256) void br_combine_f32_kernel(BrPrefillParams p, 
         }
     }
     // padded token slots: the kernels never touch them, so give them a defined value (zero)
-    const int n_pad_work = p.B * p.M * p.Nq;
+    const int n_pad_work = pv.hdr[BR_PH_PACKED] ? 0 : p.B * p.M * p.Nq;
     for (int w = blockIdx.x; w < n_pad_work; w += gridDim.x) {
         const int bm = w / p.Nq, head = w - bm * p.Nq;
         const int b = bm / p.M, mm = bm - b * p.M;

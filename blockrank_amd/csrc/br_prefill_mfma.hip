@@ -402,7 +402,7 @@ struct Prefill {
         const int row0 = it.t0 + sub * BR_RB;              // first query row of this wave, valid-relative
         const bool rb_active = row0 < len_m;
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
-        const int qtok0 = m * p.H + it.start_m;            // token index of the block's first real token
+        const int qtok0 = it.tok_m;                        // token index of the block's first real token
         const unsigned smem_lds = lds_addr_of(smem);
         const int sk_bytes = (int)p.sk_t * 2, sv_bytes = (int)p.sv_t * 2;
 
@@ -421,7 +421,7 @@ struct Prefill {
         const int first_doc_tile = (it.len0 + BR_BN - 1) / BR_BN;
         const int nprev = it.nprev;
         const int f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
-        const int own_tok0 = m * p.H + it.start_m;
+        const int own_tok0 = it.tok_m;
         int wf = it.f_lo;                                  // next tile of the walk
         int dbase = it.f_lo;
         int2 dreg = make_int2(0, 0);
@@ -445,7 +445,7 @@ struct Prefill {
             const int p_nv = it.len0 - f * BR_BN < BR_BN ? it.len0 - f * BR_BN : BR_BN;
             const int o_nv = self_end - k0 < BR_BN ? self_end - k0 : BR_BN;
             n_f = f;
-            n_tok0 = prev ? (table ? t_tok0 : it.start0 + f * BR_BN) : own_tok0 + k0;
+            n_tok0 = prev ? (table ? t_tok0 : it.tok0 + f * BR_BN) : own_tok0 + k0;
             n_nvalid = prev ? (table ? t_nv : p_nv) : o_nv;
             wf = f + 1;
             return true;
@@ -628,7 +628,7 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
         {
             int* w = reinterpret_cast<int*>(&it);
 #pragma unroll
-            for (int i = 0; i < 12; ++i) w[i] = uni(mail[cur].word[i]);
+            for (int i = 0; i < BR_ITEM_WORDS_USED; ++i) w[i] = uni(mail[cur].word[i]);
         }
         const int hg = uni(mail[cur].hg);
         if (wave == 0) pf.draw();
@@ -659,7 +659,7 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
         const BrComb c = pv.comb[ci];
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int len_m = pv.len[c.b * p.M + m];
-        const int qtok0 = m * p.H + pv.start[c.b * p.M + m];
+        const int qtok0 = pv.tok[c.b * p.M + m];
         const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
         const int row = c.t0 + sub * BR_RB + rr;
         if (row >= len_m) continue;
@@ -695,7 +695,8 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
         }
     }
     // padded token slots: the kernels never touch them, so give them a defined value (zero)
-    const int n_pad_work = p.B * p.M * p.Nq;
+    // (a packed layout has none)
+    const int n_pad_work = pv.hdr[BR_PH_PACKED] ? 0 : p.B * p.M * p.Nq;
     for (int w = blockIdx.x; w < n_pad_work; w += gridDim.x) {
         const int bm = w / p.Nq, head = w - bm * p.Nq;
         const int b = bm / p.M, mm = bm - b * p.M;

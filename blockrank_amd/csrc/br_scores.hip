@@ -61,10 +61,10 @@ struct BrScoreParams {
 // Stage the (head, row) query vectors of one workgroup into LDS as fp32, pre-multiplied by mult.
 // qs is [hc*R][D]; ok[j] says whether that row is a real token.
 template <typename T>
-__device__ void stage_queries(const BrScoreParams& p, const int* start, const int* len, int b, int head0, int nheads,
-                              float mult, float* qs, int* ok) {
+__device__ void stage_queries(const BrScoreParams& p, const BrPlanView& pv, int b, int head0, int nheads, float mult, float* qs,
+                              int* ok) {
     const int m = p.M - 1;
-    const int st = start[b * p.M + m], ln = len[b * p.M + m];
+    const int st = pv.start[b * p.M + m], ln = pv.len[b * p.M + m], tk = pv.tok[b * p.M + m];
     for (int idx = threadIdx.x; idx < nheads * p.R * p.D; idx += blockDim.x) {
         int j = idx / p.D, d = idx - j * p.D;
         int h = j / p.R, r = j - h * p.R;
@@ -72,7 +72,7 @@ __device__ void stage_queries(const BrScoreParams& p, const int* start, const in
         bool v = pos >= st && pos < st + ln;
         float x = 0.f;
         if (v) x = (float)reinterpret_cast<const T*>(p.q)[(long long)b * p.sq_b + (long long)(head0 + h) * p.sq_h +
-                                                         (long long)(m * p.H + pos) * p.sq_t + d];
+                                                         (long long)(tk + pos - st) * p.sq_t + d];
         qs[j * p.D + d] = x * mult;
         if (d == 0) ok[j] = v;
     }
@@ -118,12 +118,12 @@ __global__ __launch_bounds__(256) void br_doc_partial_kernel(BrScoreParams p) {
     const int nheads = (hchunk + 1) * p.hc <= G ? p.hc : G - hchunk * p.hc;
     const int nq = nheads * p.R;
     const int docs = p.M - 2;
-    stage_queries<T>(p, pv.start, pv.len, b, head0, nheads, p.scale * kLog2e, qs, ok);
+    stage_queries<T>(p, pv, b, head0, nheads, p.scale * kLog2e, qs, ok);
     __syncthreads();
     const int blk = doc + 1;
     const int st = pv.start[b * p.M + blk], ln = pv.len[b * p.M + blk];
     const T* kbase = reinterpret_cast<const T*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h +
-                     (long long)(blk * p.H + st) * p.sk_t;
+                     (long long)pv.tok[b * p.M + blk] * p.sk_t;
     float mx[kQR], sm[kQR];
 #pragma unroll
     for (int j = 0; j < kQR; ++j) {
@@ -360,16 +360,24 @@ __global__ __launch_bounds__(256) void br_last_logits_kernel(BrScoreParams p) {
     const int nheads = (hchunk + 1) * p.hc <= G ? p.hc : G - hchunk * p.hc;
     const int nq = nheads * p.R;
     const int S = p.M * p.H;
-    stage_queries<T>(p, pv.start, pv.len, b, head0, nheads, p.scale, qs, ok);
+    stage_queries<T>(p, pv, b, head0, nheads, p.scale, qs, ok);
     __syncthreads();
     const int key = blockIdx.x * blockDim.x + threadIdx.x;
     if (key >= S) return;
     const int blk = key / p.H, j = key - blk * p.H;
     const int st = pv.start[b * p.M + blk], ln = pv.len[b * p.M + blk];
     const bool kvalid = j >= st && j < st + ln;
-    const T* krow = reinterpret_cast<const T*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h + (long long)key * p.sk_t;
+    // (a slot that holds no real token has no key row to read - in a packed layout not even storage;
+    // its logit is the masked value whatever the dot product would be)
+    const T* krow = reinterpret_cast<const T*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h +
+                    (long long)(pv.tok[b * p.M + blk] + j - st) * p.sk_t;
     float s[kQR];
-    key_dots<T, D>(krow, qs, nq, s);
+    if (kvalid) {
+        key_dots<T, D>(krow, qs, nq, s);
+    } else {
+#pragma unroll
+        for (int jq = 0; jq < kQR; ++jq) s[jq] = 0.f;
+    }
 #pragma unroll
     for (int jq = 0; jq < kQR; ++jq) {
         if (jq < nq) {

@@ -97,6 +97,55 @@ class TruncatedRanker:
         q, _ = rope(q, q, cos[:, S - H:], sin[:, S - H:])
         return doc_scores(q, k, mask, pos, attn.scaling, temperature=self.temperature, query_block_only=True)
 
+    @torch.no_grad()
+    def forward_packed(self, input_ids: torch.Tensor, position_ids: torch.Tensor, block_lengths: torch.Tensor, rows: torch.Tensor,
+                       H: Optional[int] = None, **layer_kwargs) -> torch.Tensor:
+        """The same forward on a packed batch (see blockrank_amd.collate): input_ids, position_ids (1, T)
+        hold the real tokens only, block_lengths (B, M) says how they split into blocks, rows (B, R)
+        are indices into the last ``num_last_queries`` positions of the query block.  The dense layers
+        then run over T tokens instead of B*M*H slots.  Returns (B, M-2) fp32 scores."""
+        base = self.base
+        B, M = block_lengths.shape
+        assert M >= 3, "ranking needs a prefix, at least one document and a query block"
+        dev = input_ids.device
+        T = input_ids.shape[-1]
+        input_ids = input_ids.reshape(1, T)
+        position_ids = position_ids.reshape(1, T)
+        hidden = base.embed_tokens(input_ids)
+        mask = BlockMask.from_lengths(block_lengths.to(dev), H=H, packed=True, dtype=hidden.dtype)
+        assert mask.total_tokens == T, "block_lengths do not sum to the number of tokens"
+        Hs = mask.H
+        h1 = self.num_last_queries if Hs >= self.num_last_queries else Hs
+        pos = (rows.to(dev) + (Hs - h1)).to(torch.int32)
+        cos_sin = base.rotary_emb(hidden, position_ids=position_ids)
+        for layer in base.layers[: self.layer_idx]:
+            hidden = layer(hidden, attention_mask=mask, position_ids=position_ids, past_key_values=None, use_cache=False,
+                           position_embeddings=cos_sin, **layer_kwargs)
+            if isinstance(hidden, tuple):
+                hidden = hidden[0]
+        layer = base.layers[self.layer_idx]
+        attn = layer.self_attn
+        rope = sys.modules[type(attn).__module__].apply_rotary_pos_emb
+        D = attn.head_dim
+        for name in ("q_norm", "k_norm"):
+            if hasattr(attn, name):
+                raise NotImplementedError(f"attention modules with {name} are not supported by the truncated driver")
+        x = layer.input_layernorm(hidden)
+        cos, sin = cos_sin
+        k = attn.k_proj(x).view(1, T, -1, D).transpose(1, 2)
+        _, k = rope(k, k, cos, sin)
+        # queries of the query blocks only, scattered to their places on the token axis (the score
+        # kernels read no other query rows, so the rest of that buffer stays unwritten)
+        flat = block_lengths.to(dev).reshape(-1).long()
+        block_of = torch.repeat_interleave(torch.arange(B * M, device=dev), flat, output_size=T)
+        idx_q = ((block_of % M) == M - 1).nonzero().squeeze(-1)
+        qc = attn.q_proj(x[:, idx_q]).view(1, idx_q.numel(), -1, D).transpose(1, 2)
+        qc, _ = rope(qc, qc, cos[:, idx_q], sin[:, idx_q])
+        Nq = qc.shape[1]
+        q_full = torch.empty((1, T, Nq, D), dtype=qc.dtype, device=dev)
+        q_full[:, idx_q] = qc.transpose(1, 2)
+        return doc_scores(q_full.transpose(1, 2), k, mask, pos, attn.scaling, temperature=self.temperature)
+
     def rank(self, *args, k: int = 10, **kwargs) -> torch.Tensor:
         """Top-k document indices (B, min(k, docs)), as scripts/eval_attn.py:150-151 takes them."""
         return rank_documents(self(*args, **kwargs), k)

@@ -60,6 +60,17 @@ int br_plan_build(const uint8_t* valid, int B, int M, int H, int Nq, int Nkv, in
 int br_plan_build_from_lengths(const int32_t* lens, int left_padded, int B, int M, int H, int Nq, int Nkv,
                                int32_t* plan, size_t plan_ints, void* stream);
 
+/* Plan for a PACKED token layout: the real tokens of all blocks of all sequences follow each other on
+ * the token axis with no padded slots (sequence 0 block 0, block 1, ..., sequence 1 block 0, ...), so
+ * q, k, v and out are (1, heads, T, D) / (1, T, heads, D) tensors with T = sum of lens and the calls
+ * below take batch strides of 0.  lens: B*M int32 real-token counts on the device; H: an upper bound
+ * of the block lengths (it sizes the plan and defines the row positions of the score calls: position
+ * H-1 is a block's last token).  Same B, M, H go to every later call.  No reference counterpart: the
+ * reference pads every block to a common H (src/blockrank/dataset.py:205-227); this is the layout of
+ * a collate function that does not. */
+int br_plan_build_packed(const int32_t* lens, int B, int M, int H, int Nq, int Nkv, int32_t* plan, size_t plan_ints,
+                         void* stream);
+
 /* Bytes of scratch br_prefill_fwd needs (split-KV partials of the query block). */
 size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D);
 
