@@ -133,12 +133,21 @@ def bench_model(args):
     ranker = br.TruncatedRanker(model, layer_idx)
     steps = args.steps if args.steps is not None else 10
     warmup = args.warmup if args.warmup is not None else 2
+    if args.padded:
+        def forward(**kw):
+            return ranker(ids, valid, pos, rows=rows, **kw)
+    else:
+        pk = br.pack_padded_batch(dict(input_ids=ids, position_ids=pos, attention_mask=valid))
+        lens_dev = pk["block_lengths"]
+
+        def forward(**kw):
+            return ranker.forward_packed(pk["input_ids"], pk["position_ids"], lens_dev, rows, H=layout.H, **kw)
     for _ in range(warmup):
-        scores = ranker(ids, valid, pos, rows=rows)
+        scores = forward()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        scores = ranker(ids, valid, pos, rows=rows)
+        scores = forward()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     assert torch.isfinite(scores).all()
@@ -150,7 +159,7 @@ def bench_model(args):
             pairs.append(profiling.EventPair())
             return iter(pairs[-1].handles)
 
-    ranker(ids, valid, pos, rows=rows, kernel_events=_Events())
+    forward(kernel_events=_Events())
     torch.cuda.synchronize()
     kern_ms = [p.elapsed_ms() for p in pairs]
     kern_avg_ms = sum(kern_ms) / len(kern_ms)
@@ -168,7 +177,8 @@ def bench_model(args):
         "config": {"workload": "Mistral-7B-shaped decoder (random init), B=8, 64-token prefix + 20 docs U[96,224] + 32-token query, "
                                "layers 0..19 in full and the score part of layer 20, bf16",
                    "name": "cfg3", "batch": B, "blocks": layout.M, "block_len": layout.H, "valid_tokens": layout.valid_tokens,
-                   "padded_tokens": B * S, "unmasked_pairs": pairs_n, "launch": "eager"},
+                   "padded_tokens": B * S, "unmasked_pairs": pairs_n, "launch": "eager",
+                   "token_layout": "padded (B, M, H)" if args.padded else "packed (real tokens only)"},
         "prefill_tok_per_s": layout.valid_tokens / (ms_per_step * 1e-3),
         "attention_ms_per_step": sum(kern_ms),
         "attention_share": sum(kern_ms) / ms_per_step,
@@ -191,6 +201,8 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
+    ap.add_argument("--padded", action="store_true",
+                    help="cfg3: feed the reference's padded (B, M, H) batch instead of the packed one")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a profiler's HBM byte counters can be "
                          "scaled against a kernel of known traffic")
