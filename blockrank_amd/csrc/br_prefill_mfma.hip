@@ -646,53 +646,63 @@ template <int D>
 __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int NW) {
     const BrGeom& ge = p.geom;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
-    const int n_units = pv.hdr[BR_PH_NCOMB] * ge.NHG * NW;
+    constexpr int CPR = D / 4;                    // float4 chunks per row = threads per row
+    constexpr int RPW = 256 / CPR;                // rows one workgroup merges at a time
+    constexpr int SUBS = BR_RB / RPW;             // such row groups per 32-row block
+    const int n_units = pv.hdr[BR_PH_NCOMB] * ge.NHG * NW * SUBS;
     const int m = p.M - 1;
     const int rows = NW * BR_RB;
-    constexpr int CPR = D / 4;                    // float4 chunks per row
-    constexpr int TPR = 8;                        // threads per row
-    const int rr = threadIdx.x / TPR, cc = threadIdx.x % TPR;
+    const int rr = threadIdx.x / CPR, cc = threadIdx.x % CPR;
     for (int u = blockIdx.x; u < n_units; u += gridDim.x) {
-        const int wave = u % NW;
-        const int w = u / NW;
+        const int subu = u % SUBS;
+        const int wave = (u / SUBS) % NW;
+        const int w = u / (SUBS * NW);
         const int ci = w / ge.NHG, hg = w - ci * ge.NHG;
         const BrComb c = pv.comb[ci];
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int len_m = pv.len[c.b * p.M + m];
         const int qtok0 = pv.tok[c.b * p.M + m];
         const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
-        const int row = c.t0 + sub * BR_RB + rr;
+        const int rloc = subu * RPW + rr;                            // row inside the 32-row block
+        const int row = c.t0 + sub * BR_RB + rloc;
         if (row >= len_m) continue;
         const int head = kvh * ge.G + hsub * ge.Gw + g;
-        const int r = wave * BR_RB + rr;
+        const int r = wave * BR_RB + rloc;
         const long long slot0 = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0) * ge.NHG + hg;
         const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
-        const float* ml = p.part_ml + (slot0 * rows + r) * 2;
-        float mmax = -INFINITY;
-#pragma unroll 4
-        for (int s = 0; s < c.nsplit; ++s) mmax = fmaxf(mmax, ml[s * sstride * 2]);
-        float l = 0.f;
-        f32x4 acc[CPR / TPR];
+        const float2* ml = reinterpret_cast<const float2*>(p.part_ml) + slot0 * rows + r;
+        const float* po = p.part_o + (slot0 * rows + r) * D + cc * 4;
+        // all loads of up to eight splits are in flight together; a thread owns one float4 of the row
+        float mmax = -INFINITY, l = 0.f;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int s0 = 0; s0 < c.nsplit; s0 += 8) {
+            float2 mls[8];
+            f32x4 ov[8];
 #pragma unroll
-        for (int j = 0; j < CPR / TPR; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const float* po = p.part_o + (slot0 * rows + r) * D;
-#pragma unroll 4
-        for (int s = 0; s < c.nsplit; ++s) {
-            const float ms = ml[s * sstride * 2];
-            const float w8 = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);
-            l += ml[s * sstride * 2 + 1] * w8;
+            for (int j = 0; j < 8; ++j) {
+                const bool on = s0 + j < c.nsplit;
+                mls[j] = on ? ml[(s0 + j) * sstride] : make_float2(-INFINITY, 0.f);
+                ov[j] = on ? *reinterpret_cast<const f32x4*>(po + (s0 + j) * sstride * D) : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            float mnew = mmax;
 #pragma unroll
-            for (int j = 0; j < CPR / TPR; ++j)
-                acc[j] += *reinterpret_cast<const f32x4*>(po + s * sstride * D + (cc + j * TPR) * 4) * w8;
+            for (int j = 0; j < 8; ++j) mnew = fmaxf(mnew, mls[j].x);
+            const float resc = mmax == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mmax - mnew);
+            l *= resc;
+            acc *= resc;
+            mmax = mnew;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float w8 = mls[j].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mls[j].x - mmax);
+                l += mls[j].y * w8;
+                acc += ov[j] * w8;
+            }
         }
         const float inv = l > 0.f ? 1.f / l : 0.f;
         __bf16* dst = reinterpret_cast<__bf16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
                       (long long)(qtok0 + row) * p.so_t;
-#pragma unroll
-        for (int j = 0; j < CPR / TPR; ++j) {
-            bf16x4 h4 = __builtin_convertvector(acc[j] * inv, bf16x4);
-            *reinterpret_cast<bf16x4*>(dst + (cc + j * TPR) * 4) = h4;
-        }
+        bf16x4 h4 = __builtin_convertvector(acc * inv, bf16x4);
+        *reinterpret_cast<bf16x4*>(dst + cc * 4) = h4;
     }
     // padded token slots: the kernels never touch them, so give them a defined value (zero)
     // (a packed layout has none)

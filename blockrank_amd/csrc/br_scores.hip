@@ -262,7 +262,52 @@ __global__ __launch_bounds__(1024) void br_doc_final_tiles_kernel(BrTileScorePar
         t0 = tbase[b * p.M + lane + 1];
         nt = (len[b * p.M + lane + 1] + BR_BN - 1) / BR_BN;
     }
-    for (int j = wave; j < NR; j += nwaves) {
+    if (small) {
+        // four (head, row) pairs of a wave at a time: all their loads are issued before the first reduction
+        constexpr int PG = 4;
+        for (int j0 = wave; j0 < NR; j0 += PG * nwaves) {
+            float2 v[PG][8];
+            bool pair_on[PG];
+#pragma unroll
+            for (int i = 0; i < PG; ++i) {
+                const int j = j0 + i * nwaves;
+                pair_on[i] = j < NR;
+                const int jj = pair_on[i] ? j : 0;
+                const int n = jj / p.R, r = jj - n * p.R;
+                int r16 = p.rows[b * p.R + r];
+                r16 = r16 < 0 ? 0 : (r16 >= p.Rw ? p.Rw - 1 : r16);
+                const int pos = p.H - p.Rw + r16;
+                const bool row_ok = pair_on[i] && pos >= st_q && pos < st_q + len_q;
+                const float2* base = reinterpret_cast<const float2*>(p.part) + (((long long)b * p.Nq + n) * p.Rw + r16) * tps;
+#pragma unroll
+                for (int t8 = 0; t8 < 8; ++t8) v[i][t8] = (row_ok && t8 < nt) ? base[t0 + t8] : make_float2(-INFINITY, 0.f);
+            }
+#pragma unroll
+            for (int i = 0; i < PG; ++i) {
+                if (!pair_on[i]) continue;
+                const int j = j0 + i * nwaves;
+                float* pr_out = p.probs ? p.probs + ((long long)b * NR + j) * docs : nullptr;
+                float mx = -INFINITY;
+#pragma unroll
+                for (int t8 = 0; t8 < 8; ++t8) mx = fmaxf(mx, v[i][t8].x);
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+                float sd = 0.f;
+#pragma unroll
+                for (int t8 = 0; t8 < 8; ++t8)
+                    if (v[i][t8].x != -INFINITY) sd += v[i][t8].y * __builtin_amdgcn_exp2f(v[i][t8].x - mx);
+                float den = sd;
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
+                if (lane < docs) {
+                    const float pr = den > 0.f ? sd / den : uniform;
+                    if (pr_out) pr_out[lane] = pr;
+                    mine[lane] += pr;
+                }
+            }
+        }
+    }
+    for (int j = wave; j < NR && !small; j += nwaves) {
         const int n = j / p.R, r = j - n * p.R;
         int r16 = p.rows[b * p.R + r];
         r16 = r16 < 0 ? 0 : (r16 >= p.Rw ? p.Rw - 1 : r16);
@@ -270,28 +315,7 @@ __global__ __launch_bounds__(1024) void br_doc_final_tiles_kernel(BrTileScorePar
         const bool row_ok = pos >= st_q && pos < st_q + len_q;
         const float2* base = reinterpret_cast<const float2*>(p.part) + (((long long)b * p.Nq + n) * p.Rw + r16) * tps;
         float* pr_out = p.probs ? p.probs + ((long long)b * NR + j) * docs : nullptr;
-        if (small) {
-            float2 v[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = (row_ok && i < nt) ? base[t0 + i] : make_float2(-INFINITY, 0.f);
-            float mx = -INFINITY;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) mx = fmaxf(mx, v[i].x);
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-            float sd = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (v[i].x != -INFINITY) sd += v[i].y * __builtin_amdgcn_exp2f(v[i].x - mx);
-            float den = sd;
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
-            if (lane < docs) {
-                const float pr = den > 0.f ? sd / den : uniform;
-                if (pr_out) pr_out[lane] = pr;
-                mine[lane] += pr;
-            }
-        } else {
+        {
             float mx = -INFINITY;
             if (row_ok)
                 for (int d = lane; d < docs; d += 64) {
