@@ -39,6 +39,10 @@ SIGNATURES = {
     "br_prefill_fwd_scores": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t,
                                       c_int, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "br_prefill_fp8qk_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int64]),
+    "br_prefill_fwd_fp8qk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_void_p, c_size_t,
+                                     c_int, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),
     "br_doc_scores_from_partials": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                                             c_void_p, c_void_p, c_void_p]),
     "br_doc_scores_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),

@@ -229,6 +229,7 @@ def blockrank_attention(
     *,
     kernel_events=None,
     score_rows: int = 0,
+    qk_fp8: bool = False,
 ):
     """Block-sparse prefill attention.  query (B, Nq, S, D), key/value (B, Nkv, S, D) with any
     (batch, head, token) strides; block_mask a BlockMask, a (B, M, H) bool tensor, or the reference's
@@ -240,7 +241,11 @@ def blockrank_attention(
 
     score_rows > 0 (bf16, at least one document block): the same kernel pass also leaves the per-tile
     score partials of the query block's last score_rows positions, and the call returns
-    (out, partials); ``doc_scores_from_partials`` turns them into per-document scores."""
+    (out, partials); ``doc_scores_from_partials`` turns them into per-document scores.
+
+    qk_fp8 (bf16 inputs, head dim 128): Q K^T is computed in fp8 e4m3 with per-(sequence, head) absmax
+    scales, P V stays bf16 - the reduced-precision variant for ranking (scores stay within 5e-3
+    relative of the fp32 result)."""
     if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
         block_mask = BlockMask(block_mask, query.dtype)
     bm = _as_block_mask(block_mask)
@@ -274,6 +279,22 @@ def blockrank_attention(
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         out_strides = _lib._I64x3(0 if packed else S * Nq * D, D, Nq * D)
         ev0, ev1 = kernel_events if kernel_events is not None else (None, None)
+        if qk_fp8:
+            if query.dtype != torch.bfloat16 or D != 128:
+                raise NotImplementedError("the fp8 Q K^T variant takes bfloat16 inputs with head dim 128")
+            tokens = S if packed else B * S
+            f8_bytes = lib.br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, tokens)
+            ws8 = torch.empty(max(f8_bytes, 16), dtype=torch.uint8, device=dev)
+            part, sp_bytes = None, 0
+            if score_rows > 0:
+                sp_bytes = lib.br_score_partials_bytes(B, Nq, M, H, score_rows)
+                part = torch.empty(max(sp_bytes // 4, 4), dtype=torch.float32, device=dev)
+            _lib.check(lib.br_prefill_fwd_fp8qk(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
+                _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed), out_strides, float(scaling),
+                tokens, ws8.data_ptr(), f8_bytes, score_rows, part.data_ptr() if part is not None else None, sp_bytes,
+                _stream_ptr(dev), ev0, ev1))
+            return (out, part) if score_rows > 0 else out
         if score_rows > 0:
             sp_bytes = lib.br_score_partials_bytes(B, Nq, M, H, score_rows)
             part = torch.empty(max(sp_bytes // 4, 4), dtype=torch.float32, device=dev)
@@ -482,6 +503,7 @@ def blockrank_attention_forward(
     LastBlockScores handle (scaled logits, the eager/Triton convention); pass
     ``materialize_scores=True`` or set BLOCKRANK_AMD_DENSE_SCORES=1 for the fp32 tensor itself, and
     ``unscaled_scores=True`` for the literal SDPA function's unscaled variant (:537, :643).
+    ``qk_fp8=True`` (or BLOCKRANK_AMD_QK_FP8=1) computes Q K^T in fp8 e4m3 (see blockrank_attention).
     """
     assert attention_mask is not None, "BlockRank attention requires an attention mask"
     bm = _as_block_mask(attention_mask)
@@ -506,8 +528,9 @@ def blockrank_attention_forward(
     scaled = not kwargs.get("unscaled_scores", False)
     fuse = want and scaled and fused_scores_supported(query, bm) and not _env_flag("BLOCKRANK_AMD_SEPARATE_SCORES")
 
+    qk_fp8 = bool(kwargs.get("qk_fp8", False)) or _env_flag("BLOCKRANK_AMD_QK_FP8")
     out = blockrank_attention(query, key, value, bm, scaling, kernel_events=kwargs.get("kernel_events", None),
-                              score_rows=R if fuse else 0)
+                              score_rows=R if fuse else 0, qk_fp8=qk_fp8)
     partials = None
     if fuse:
         out, partials = out

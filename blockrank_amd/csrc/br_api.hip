@@ -16,6 +16,11 @@ int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
                          float* probs, const long long* sq, const long long* sk, int B, int Nq, int Nkv, int M, int H, int D,
                          int R, int T, float scale, float out_scale, int dtype, hipStream_t stream);
+int br_launch_prefill_fp8qk(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
+                            hipEvent_t ev_start, hipEvent_t ev_stop);
+void br_launch_quantize_fp8(const void* q, const void* k, const int* plan, void* q8, void* k8, unsigned* amax, float* scales,
+                            const long long* sq, const long long* sk, long long q8_b, long long q8_h, long long k8_b, long long k8_h,
+                            int B, int Nq, int Nkv, int M, int H, int D, hipStream_t stream);
 int br_launch_doc_scores_tiles(const float* part, const int* plan, const int* rows, float* scores, float* probs, int B, int Nq,
                                int M, int H, int R, int Rw, float out_scale, hipStream_t stream);
 int br_launch_last_logits(const void* q, const void* k, const int* plan, const int* rows, float* logits, const long long* sq,
@@ -172,10 +177,21 @@ size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows) {
     return (size_t)B * Nq * score_rows * br_plan_tps(M, H) * 2 * sizeof(float);
 }
 
+static size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int64_t tokens) {
+    const size_t base = br_prefill_workspace_bytes(B, Nq, Nkv, D);
+    if (base == 0 || tokens <= 0) return 0;
+    return up256(base) + up256((size_t)Nq * tokens * D) + up256((size_t)Nkv * tokens * D) + 2 * up256((size_t)B * (Nq + Nkv) * 4);
+}
+
+// fp8_tokens > 0: Q K^T in fp8 (inputs bf16, quantised into the workspace first); it is the length of the
+// token axis summed over the batch (B*M*H padded slots, or the packed token count).
 static int prefill_impl(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
                         int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                         const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
-                        void* stream, void* ev_start, void* ev_stop, int score_rows, float* score_part, size_t score_part_bytes) {
+                        void* stream, void* ev_start, void* ev_stop, int score_rows, float* score_part, size_t score_part_bytes,
+                        int64_t fp8_tokens = 0) {
     int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
     if (rc) return rc;
     if (score_part) {
@@ -195,7 +211,9 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     BrGeom g;
     int nw;
     make_geom(Nq, Nkv, &g, &nw);
-    const size_t need = br_prefill_workspace_bytes(B, Nq, Nkv, D);
+    if (fp8_tokens > 0 && (dtype != BR_DTYPE_BF16 || D != 128))
+        return fail(BR_ERR_ARG, "the fp8 Q K^T variant takes bf16 inputs with head dim 128");
+    const size_t need = fp8_tokens > 0 ? br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, fp8_tokens) : br_prefill_workspace_bytes(B, Nq, Nkv, D);
     if (!workspace || workspace_bytes < need) return fail(BR_ERR_SPACE, "workspace holds %zu bytes, %zu needed", workspace_bytes, need);
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
@@ -214,13 +232,37 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     p.scale_log2 = scale * 1.4426950408889634f;
     p.score_part = score_part;
     p.score_R = score_part ? score_rows : 0;
+    p.qk_scales = nullptr;
     int combine_grid = br_plan_max_comb(B) * g.NHG;
     if (combine_grid < B * M) combine_grid = B * M;
     if (combine_grid > 4 * n_cu) combine_grid = 4 * n_cu;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipEvent_t e0 = static_cast<hipEvent_t>(ev_start), e1 = static_cast<hipEvent_t>(ev_stop);
-    int lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1)
+    int lrc;
+    if (fp8_tokens > 0) {
+        const bool packed = q_strides[0] == 0;
+        const long long stot = packed ? fp8_tokens : fp8_tokens / B;        // tokens per batch entry of q8/k8
+        char* w = static_cast<char*>(workspace) + up256(br_prefill_workspace_bytes(B, Nq, Nkv, D));
+        void* q8 = w;
+        w += up256((size_t)Nq * fp8_tokens * D);
+        void* k8 = w;
+        w += up256((size_t)Nkv * fp8_tokens * D);
+        unsigned* amax = reinterpret_cast<unsigned*>(w);
+        w += up256((size_t)B * (Nq + Nkv) * 4);
+        float* scales = reinterpret_cast<float*>(w);
+        const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]}, sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
+        const long long q8_h = stot * D, k8_h = stot * D;
+        const long long q8_b = packed ? 0 : (long long)Nq * q8_h, k8_b = packed ? 0 : (long long)Nkv * k8_h;
+        br_launch_quantize_fp8(q, k, plan, q8, k8, amax, scales, sq, sk, q8_b, q8_h, k8_b, k8_h, B, Nq, Nkv, M, H, D, s);
+        p.q = q8; p.k = k8;
+        p.sq_b = q8_b; p.sq_h = q8_h; p.sq_t = D;
+        p.sk_b = k8_b; p.sk_h = k8_h; p.sk_t = D;
+        p.qk_scales = scales;
+        lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1);
+    } else {
+        lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1)
                                      : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s, e0, e1);
+    }
     if (lrc) return fail(BR_ERR_ARG, "no kernel for head dim %d with %d query heads per kv head", D, g.G);
     return check_launch("prefill launch");
 }
@@ -248,6 +290,16 @@ int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out
     if (!score_part) return fail(BR_ERR_ARG, "score_part must be provided");
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
                         workspace, workspace_bytes, stream, ev_start, ev_stop, score_rows, score_part, score_part_bytes);
+}
+
+int br_prefill_fwd_fp8qk(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                         int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                         const int64_t* out_strides, float scale, int64_t tokens, void* workspace, size_t workspace_bytes,
+                         int score_rows, float* score_part, size_t score_part_bytes, void* stream, void* ev_start, void* ev_stop) {
+    if (tokens <= 0) return fail(BR_ERR_ARG, "tokens must be positive (got %lld)", (long long)tokens);
+    return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale,
+                        BR_DTYPE_BF16, workspace, workspace_bytes, stream, ev_start, ev_stop, score_rows, score_part,
+                        score_part_bytes, tokens);
 }
 
 int br_doc_scores_from_partials(const float* score_part, const int32_t* plan, const int32_t* rows, int R, int score_rows, int B,

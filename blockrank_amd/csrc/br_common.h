@@ -245,4 +245,7 @@ struct BrPrefillParams {
     // key tile, in the order of the sequence's tile descriptors.  Null: not wanted.
     float* score_part;
     int score_R;
+    // fp8 Q/K variant: q and k then point at e4m3 tensors (strides in elements = bytes) and qk_scales
+    // holds the dequantisation scales, [B][Nq] for Q followed by [B][Nkv] for K.  Null otherwise.
+    const float* qk_scales;
 };

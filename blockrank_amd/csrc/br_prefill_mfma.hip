@@ -1,731 +1,11 @@
-// Block-sparse prefill attention for gfx950, 16-bit inputs (bf16), fp32 softmax and accumulation.
-//
-// What it computes (reference: sdpa_blockrank_attention_forward, blockrank_std_attention.py:503-650):
-// for every real query token, softmax(scale * q.k) over the keys it may see, times V, where the
-// prefix block sees itself causally, a document sees the prefix in full plus itself causally, and
-// the query block sees every earlier block in full plus itself causally.  Padded slots are neither
-// read nor computed (the reference leaves an unspecified average there and never consumes it); the
-// finish kernel sets them to zero.
-//
-// How: a persistent grid pulls work items (query tile x key-walk range) from the request plan.  A
-// workgroup of NW waves stages each 64-key K tile and V^T tile in LDS once and every wave - one
-// 32-row block of one query head of the kv head's group - consumes them, so K/V are read once per
-// head group, not once per query head.  Per wave and tile:
-//   S^T = K Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q^T held in registers
-//   online softmax   each lane owns one query row and half of the tile's keys, so the row max / sum
-//                    need one cross-lane exchange (lane ^ 32) and the O rescale is a per-lane scalar
-//   O^T += V^T P^T   A = V^T rows from LDS, B = P^T straight from the S^T accumulators: the K rows
-//                    are assigned to MFMA rows in a permuted order chosen so that the accumulator
-//                    registers a lane ends up holding are exactly the 8 consecutive keys the next
-//                    MFMA's B operand wants, so P never travels through LDS.
-//
-// Data movement: K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4, 64
-// lanes x 16 bytes per instruction, no staging registers); which 16-byte piece of which row a lane
-// fetches is free, and that freedom provides both the row permutation and the swizzles below.  V is
-// kept row-major ([key][dim]) and read with ds_read_b64_tr_b16, which hands each lane four
-// consecutive keys of one dim - the MFMA A-operand layout of V^T - so V is never transposed by ALU code.
-//
-// LDS layouts (row = 2*D bytes, 16-byte chunks; reads are bank-conflict free):
-//   K    row r of each 32-row half holds key swap23(r) (bits 2 and 3 of the index exchanged) so that
-//        MFMA row = LDS row; chunk c of row r sits at chunk c ^ (r & 7).
-//   V    row = key; chunk c of row r sits at chunk c ^ ((r & 3) << 1).
-#include "br_common.h"
+// bf16 instances of the block-sparse prefill kernel (the templates live in br_prefill_mfma_impl.h).
+#include "br_prefill_mfma_impl.h"
 
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-
-template <int D>
-struct Smem {
-    static constexpr int rowB = D * 2;                     // bytes per K or V row
-    static constexpr int kBytes = BR_BN * rowB;
-    static constexpr int stageBytes = 2 * kBytes;          // K tile then V tile
-    static constexpr int eRow = D + 8;                     // epilogue tile: [32 rows][eRow] per wave
-    static constexpr int eBytesPerWave = BR_RB * eRow * 2;
-    static constexpr int total(int nw) {
-        int a = 2 * stageBytes, b = nw * eBytesPerWave;
-        return a > b ? a : b;
-    }
-};
-
-__device__ inline uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
-__device__ inline bf16x8 as_bf16x8(uint4 u) {
-    union { uint4 u; bf16x8 v; } c;
-    c.u = u;
-    return c.v;
-}
-__device__ inline int uni(int x) { return __builtin_amdgcn_readfirstlane(x); }
-
-// 64 lanes x 16 bytes from global memory (uniform base + per-lane byte offset) into LDS at
-// lds_addr + lane * 16.  Issued through asm so that the compiler does not make later LDS reads of
-// other buffers wait for it; completion is awaited explicitly (vm_wait_all) before the barrier that
-// publishes the tile.
-__device__ inline void dma16(const void* base, int byte_off, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
-}
-__device__ inline void vm_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-__device__ inline unsigned lds_addr_of(const void* p) {
-    return (unsigned)(size_t)(__attribute__((address_space(3))) const void*)p;
-}
-
-// Exchange bits 2 and 3.  MFMA row r of a 32-key half tile carries key swap23(r): with the 32x32
-// accumulator layout (lane = column + 32*h; register v is row 8*(v/4) + 4*h + v%4) registers
-// 8*jp .. 8*jp+7 of lane half h then hold keys 16*jp + 8*h + 0..7, which is the B-operand layout of
-// the P^T V product.
-__device__ inline int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
-
-// Descriptor prefetch, run by wave 0 while the workgroup computes an item: the ticket for the next
-// item is drawn at the start of the current one; after the first key tile the 64-byte item it names
-// is requested, and at the end of the item it is published through LDS.  Each step consumes a value
-// whose load was issued a whole tile earlier, so the chain ticket -> item costs the item's critical
-// path nothing (an item with a single tile finishes the chain at its end, waiting as needed).
-//
-// A workgroup draws from the global queue, then from the queue of its XCD (by workgroup index: the
-// hardware deals workgroups round robin to the XCDs), and is done when both are dry.  It does not look into the other XCDs' queues: the plan cuts the work into eight runs of
-// equal estimated size, and polling other queues' counters at the end of the kernel (with atomics
-// or with loads) was measured to stretch the memory waits of every workgroup still working from
-// 0.1 to 5-15 us.
-struct BrDescMail {      // layout of one LDS mailbox
-    int word[BR_ITEM_INTS];
-    int hg;
-    int valid;
-    int pad[2];
-};
-
-struct BrPrefetch {
-    int* hdr;
-    const BrPlanView* pv;
-    int NHG, lane;
-    int xq, ng;    // this workgroup serves the XCD queues xq, xq + ng, ... (ng = 8 unless the grid is smaller)
-    int qk, qend;  // step in the queue order: 0 global queue, 1.. own queues, qend done
-    int counts;    // lane j: tickets of queue j
-    int qoffs;     // lane j: index of queue j's first item
-    int scounts;   // lane j: tickets of queue j handed out statically (one per workgroup, see init)
-    int t_next;    // ticket drawn from the queue at step qk (lane 0), or -1
-    int stage;     // 0 ticket drawn, 2 item requested, 9 nothing in flight
-    int word, hg;
-
-    // The first ticket of every workgroup is fixed by its index, with no atomic (512 workgroups
-    // drawing from one counter at the same moment queue up for microseconds): workgroups 0..SG-1
-    // take the global queue's tickets 0..SG-1; the others take, in index order, the first tickets of
-    // the queue blockIdx & 7 (workgroups are dealt round robin to the XCDs, so this is normally the
-    // queue of the XCD they run on; if it is not, only locality is lost).  The counters therefore
-    // count the tickets drawn after the static ones.
-    __device__ void init(int* hdr_, const BrPlanView* pv_, int NHG_, int lane_) {
-        hdr = hdr_; pv = pv_; NHG = NHG_; lane = lane_;
-        counts = lane < BR_NQUEUES ? hdr[BR_PH_QCOUNT + lane] * NHG : 0;
-        qoffs = lane < BR_NQUEUES ? hdr[BR_PH_QOFF + lane] : 0;
-        const int grid = gridDim.x, me = blockIdx.x;
-        // Queue ownership goes by workgroup index, not by the XCD id the hardware reports: every queue
-        // then has its workgroups whatever the placement is, so all work is done in any case.
-        ng = grid < 8 ? grid : 8;
-        xq = me % ng;
-        qend = 1 + (8 - xq + ng - 1) / ng;
-        const int cg = __builtin_amdgcn_readlane(counts, BR_GLOBAL_QUEUE);
-        const int SG = grid < 8 ? 0 : (cg < grid ? cg : grid);      // (no static tickets on a tiny grid)
-        const int first = SG + ((lane - SG) & 7);                   // lane j < 8: first workgroup of queue j
-        const int nwg = first < grid ? (grid - 1 - first) / 8 + 1 : 0;
-        scounts = lane < 8 ? (nwg < counts ? nwg : counts) : (lane == BR_GLOBAL_QUEUE ? SG : 0);
-        if (grid < 8) scounts = 0;
-        qk = SG == cg ? 1 : 0;      // every global ticket handed out already: start at the XCD's own queue
-        t_next = -1;
-        stage = 9;
-        word = hg = 0;
-        int q = -1, t = 0;
-        if (me < SG) {
-            q = BR_GLOBAL_QUEUE;
-            t = me;
-        } else if (grid >= 8) {
-            const int x = me & 7;
-            const int r = (me - __builtin_amdgcn_readlane(first, x)) >> 3;
-            if (r < __builtin_amdgcn_readlane(scounts, x)) {
-                q = x;
-                t = r;
-            }
-        }
-        if (q >= 0) request(q, t);
-    }
-    __device__ int queue_now() const { return qk == 0 ? BR_GLOBAL_QUEUE : xq + (qk - 1) * ng; }
-    __device__ void request(int q, int t) {   // ask for the item that ticket t of queue q names
-        const int li = t / NHG;
-        hg = t - li * NHG;
-        const int idx = __builtin_amdgcn_readlane(qoffs, q) + li;
-        word = reinterpret_cast<const int*>(pv->items + idx)[lane & (BR_ITEM_INTS - 1)];
-        stage = 2;
-    }
-    __device__ void draw() {   // at the start of an item
-        t_next = -1;
-        stage = 9;
-        if (qk < qend) {
-            if (lane == 0) t_next = atomicAdd(&hdr[BR_PH_QTICKET + queue_now()], 1);
-            stage = 0;
-        }
-    }
-    __device__ void step() {   // once per key tile, after the tile's arithmetic
-        if (stage == 0) {
-            const int q = queue_now();
-            const int t = __builtin_amdgcn_readfirstlane(t_next) + __builtin_amdgcn_readlane(scounts, q);
-            if (t < __builtin_amdgcn_readlane(counts, q)) {
-                request(q, t);
-            } else {
-                stage = 9;
-                ++qk;          // that queue is dry for good
-            }
-        }
-    }
-    // Nothing in flight: draw now, from the global queue and then the own one.
-    __device__ bool find_work() {
-        while (qk < qend) {
-            const int q = queue_now();
-            int t = 0;
-            if (lane == 0) t = atomicAdd(&hdr[BR_PH_QTICKET + q], 1);
-            t = __builtin_amdgcn_readfirstlane(t) + __builtin_amdgcn_readlane(scounts, q);
-            if (t < __builtin_amdgcn_readlane(counts, q)) {
-                request(q, t);
-                return true;
-            }
-            ++qk;
-        }
-        return false;
-    }
-    __device__ void publish(BrDescMail* mail) {   // at the end of an item (and once before the first)
-        if (stage == 0) step();
-        if (stage == 9 && !find_work()) {
-            if (lane == 0) mail->valid = 0;
-            return;
-        }
-        if (lane < BR_ITEM_INTS) mail->word[lane] = word;
-        if (lane == 0) {
-            mail->hg = hg;
-            mail->valid = 1;
-        }
-    }
-};
-
-template <int D, int NW>
-struct Prefill {
-    static constexpr int CPR = D / 8;                      // 16-byte chunks per K/V row
-    static constexpr int NI = BR_BN * CPR / 64;            // DMA instructions per K (or V) tile
-    static constexpr int JK = (NI + NW - 1) / NW;          // per wave
-    using SM = Smem<D>;
-
-    // Per-lane constants, fixed for the whole kernel.
-    // With 4 or 8 waves the DMA pieces of one lane are a whole number of 16-row groups apart, so one
-    // offset plus a uniform step describes them all; otherwise each piece keeps its own offset.
-    static constexpr bool UNIFORM_STEP = (NW == 4 || NW == 8);
-    static constexpr int JO = UNIFORM_STEP ? 1 : JK;
-    static constexpr int STEP_ROWS = NW * 64 / CPR;        // rows between consecutive pieces of a wave
-    struct Lane {
-        int koff[JO], voff[JO];    // global byte offsets inside a tile of this lane's DMA pieces
-        int krd;                   // LDS byte offset of the K operand read of chunk 0; chunk c is krd ^ (c << 5)
-        int vrd[D / 32];           // LDS byte offsets of the V^T operand reads, one per 32-dim block
-    };
-
-    static __device__ inline Lane make_lane(const BrPrefillParams& p, int wave, int lane) {
-        Lane L;
-#pragma unroll
-        for (int j = 0; j < JO; ++j) {
-            const int slot = (wave + NW * j) * 64 + lane;
-            const int prow = slot / CPR, cp = slot - prow * CPR;
-            const int kkey = (prow & 32) | swap23(prow & 31);
-            L.koff[j] = kkey * (int)p.sk_t * 2 + ((cp ^ (prow & 7)) << 4);
-            L.voff[j] = prow * (int)p.sv_t * 2 + ((cp ^ ((prow & 3) << 1)) << 4);
-        }
-        const int ln = lane & 31, lh = lane >> 5;
-        L.krd = ln * SM::rowB + ((lh ^ (ln & 7)) << 4);
-        // transposing read: within a group of 16 lanes, lane s points at key (s >> 2), dims 4 * (s & 3)
-        const int s = lane & 15, ln_hi = (lane >> 4) & 1;
-        const int cl = (2 * ln_hi + ((s & 3) >> 1)) ^ ((s >> 2) << 1);
-#pragma unroll
-        for (int d = 0; d < D / 32; ++d)
-            L.vrd[d] = SM::kBytes + (8 * lh + (s >> 2)) * SM::rowB + (((4 * d) ^ cl) << 4) + (s & 1) * 8;
-        return L;
-    }
-
-    // Start the DMA of one K/V tile into a stage.  kt / vt point at the tile's first row (uniform).
-    // lane_l is the lane index as an opaque value of the current loop iteration: the row arithmetic of
-    // the partial-tile path is then redone where it is needed (it is rare) instead of being kept in
-    // registers across the whole key loop.
-    static __device__ inline void issue_tile(const Lane& L, int wave, int lane_l, const __bf16* kt, const __bf16* vt, int sk_bytes,
-                                             int sv_bytes, int nvalid, unsigned stage_lds) {
-        if (nvalid == BR_BN) {
-#pragma unroll
-            for (int j = 0; j < JK; ++j) {
-                const int q = wave + NW * j;
-                if (NI % NW == 0 || q < NI) {
-                    if (UNIFORM_STEP) {
-                        dma16(reinterpret_cast<const char*>(kt) + j * STEP_ROWS * sk_bytes, L.koff[0], stage_lds + q * 1024);
-                        dma16(reinterpret_cast<const char*>(vt) + j * STEP_ROWS * sv_bytes, L.voff[0], stage_lds + SM::kBytes + q * 1024);
-                    } else {
-                        dma16(kt, L.koff[j], stage_lds + q * 1024);
-                        dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
-                    }
-                }
-            }
-        } else {
-            // rows past the tile's real keys are not fetched: the LDS rows keep older (finite) data,
-            // which the kernel masks (K) or multiplies by exact zeros (V)
-#pragma unroll
-            for (int j = 0; j < JK; ++j) {
-                const int q = wave + NW * j;
-                if (NI % NW == 0 || q < NI) {
-                    const int prow = (q * 64 + lane_l) / CPR;                   // V row of this piece
-                    const int kkey = (prow & 32) | swap23(prow & 31);          // K row of this piece
-                    if (UNIFORM_STEP) {
-                        if (kkey < nvalid)
-                            dma16(reinterpret_cast<const char*>(kt) + j * STEP_ROWS * sk_bytes, L.koff[0], stage_lds + q * 1024);
-                        if (prow < nvalid)
-                            dma16(reinterpret_cast<const char*>(vt) + j * STEP_ROWS * sv_bytes, L.voff[0], stage_lds + SM::kBytes + q * 1024);
-                    } else {
-                        if (kkey < nvalid) dma16(kt, L.koff[j], stage_lds + q * 1024);
-                        if (prow < nvalid) dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
-                    }
-                }
-            }
-        }
-    }
-
-    static __device__ inline bf16x8 read_k(const char* stage, const Lane& L, int kb, int c) {
-        return as_bf16x8(ld16(stage + kb * 32 * SM::rowB + (L.krd ^ (c << 5))));
-    }
-    // V^T operand for dims 32d + (lane & 31), keys 16*c2 + 8*lh + 0..7: two transposing reads
-    static __device__ inline bf16x8 read_vt(const char* stage, const Lane& L, int d, int c2) {
-        const char* vp = stage + L.vrd[d] + c2 * 16 * SM::rowB;
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)vp);
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)(vp + 4 * SM::rowB));
-        union { s16x8 s8; bf16x8 b8; } a;
-        a.s8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        return a.b8;
-    }
-
-    // One wave, one 64-key tile already in LDS: S^T = K Q^T, online softmax, O^T += V^T P^T.
-    // NKB 32-key halves are computed (the second half is skipped when no row of the wave can see it);
-    // with MASK, keys >= lim (per row: the tile's real keys and the diagonal) are excluded.  Every
-    // variant is one straight-line block with the LDS operand reads issued ahead of their use.
-    template <int NKB, bool MASK>
-    static __device__ inline void compute_tile(const char* stage, const Lane& L, const bf16x8 (&qf)[D / 16], f32x16 (&o)[D / 32],
-                                               float& m_run, float& l_run, float scale_log2, int lim, int lh, float& psum_out) {
-        constexpr int NC = D / 16, ND = D / 32, NR = NKB * NC;
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        f32x16 s[NKB];
-        {
-            // read i: half i % NKB, chunk i / NKB - the halves alternate so that consecutive MFMAs are
-            // independent; reads run 4 ahead
-            bf16x8 ka[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ka[i] = read_k(stage, L, i % NKB, i / NKB);
-#pragma unroll
-            for (int kb = 0; kb < NKB; ++kb) s[kb] = zero;
-#pragma unroll
-            for (int i = 0; i < NR; ++i) {
-                const bf16x8 a = ka[i & 3];
-                if (i + 4 < NR) ka[i & 3] = read_k(stage, L, (i + 4) % NKB, (i + 4) / NKB);
-                s[i % NKB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[i / NKB], s[i % NKB], 0, 0, 0);
-            }
-        }
-        // first V^T operands: their LDS latency passes under the softmax arithmetic
-        bf16x8 va[ND];
-#pragma unroll
-        for (int d = 0; d < ND; ++d) va[d] = read_vt(stage, L, d, 0);
-        if (MASK) {
-#pragma unroll
-            for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int key = kb * 32 + 16 * (v >> 3) + 8 * lh + (v & 7);
-                    if (key >= lim) s[kb][v] = -INFINITY;
-                }
-        }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        // Lazy rescale: the running max is only raised (and O, l rescaled) when some row's max grew by
-        // more than 2^8; otherwise exponentials are taken against the older max, which changes nothing
-        // in the final quotient and keeps them below 2^8.
-        const float m_new = fmaxf(m_run, mx * scale_log2);
-        if (__builtin_amdgcn_ballot_w64(m_new - m_run > 8.f) != 0) {
-            const float m_sub = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_sub);
-            m_run = m_new;
-            l_run *= alpha;
-#pragma unroll
-            for (int d = 0; d < ND; ++d)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
-        }
-        const float m_sub = m_run == -INFINITY ? 0.f : m_run;
-        float psum = 0.f;
-        bf16x8 pf[2 * NKB];
-#pragma unroll
-        for (int c2 = 0; c2 < 2 * NKB; ++c2) {
-            f32x8 t;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                t[e] = __builtin_amdgcn_exp2f(s[c2 >> 1][8 * (c2 & 1) + e] * scale_log2 - m_sub);
-                psum += t[e];
-            }
-            pf[c2] = __builtin_convertvector(t, bf16x8);
-        }
-        l_run += psum;
-        psum_out = psum;
-#pragma unroll
-        for (int c2 = 0; c2 < 2 * NKB; ++c2) {
-#pragma unroll
-            for (int d = 0; d < ND; ++d) {
-                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d], pf[c2], o[d], 0, 0, 0);
-                if (c2 + 1 < 2 * NKB) va[d] = read_vt(stage, L, d, c2 + 1);
-            }
-        }
-    }
-
-    static __device__ void run_item(const BrPrefillParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem,
-                                    const Lane& L, BrPrefetch& pf) {
-        const int tid = threadIdx.x;
-        const int wave = uni(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
-        const BrGeom& ge = p.geom;
-        const int T = ge.tpb * BR_RB;
-        const int b = it.b, m = it.m;
-        const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
-        const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
-        const int head = kvh * ge.G + hsub * ge.Gw + g;
-        const int len_m = it.len_m;
-        const int row0 = it.t0 + sub * BR_RB;              // first query row of this wave, valid-relative
-        const bool rb_active = row0 < len_m;
-        const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
-        const int qtok0 = it.tok_m;                        // token index of the block's first real token
-        const unsigned smem_lds = lds_addr_of(smem);
-        const int sk_bytes = (int)p.sk_t * 2, sv_bytes = (int)p.sv_t * 2;
-
-        const __bf16* kbase = reinterpret_cast<const __bf16*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h;
-        const __bf16* vbase = reinterpret_cast<const __bf16*>(p.v) + (long long)b * p.sv_b + (long long)kvh * p.sv_h;
-
-        // The walk over the item's key tiles needs no memory lookups inside the loop: a document's only
-        // earlier block is the prefix (described by the item itself); a query-block item keeps the
-        // descriptors of its earlier-block tiles in lane registers (lane i = tile dbase + i) and reads
-        // them with readlane.  Every quantity is a scalar computed with selects (no tile structs: they
-        // would end up in scratch memory, and a scratch load waits for the tile DMAs in flight).
-        const int2* tiles_b = pv.tiles + (size_t)b * pv.tps;
-        const bool table = it.pe > 1;
-        // only query-block items of a sequence with documents emit score partials, for document tiles
-        const bool emit_scores = p.score_part != nullptr && table && m == p.M - 1;
-        const int first_doc_tile = (it.len0 + BR_BN - 1) / BR_BN;
-        const int nprev = it.nprev;
-        const int f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
-        const int own_tok0 = it.tok_m;
-        int wf = it.f_lo;                                  // next tile of the walk
-        int dbase = it.f_lo;
-        int2 dreg = make_int2(0, 0);
-        if (table && dbase + lane < nprev) dreg = tiles_b[dbase + lane];
-        // tile state: index in the walk (earlier-block tiles come first, f < nprev; then the block's
-        // own tiles), first token, real keys
-        int c_f = 0, c_tok0 = 0, c_nvalid = 0;
-        int n_f = 0, n_tok0 = 0, n_nvalid = 0;
-        auto fetch = [&]() -> bool {
-            const int f = wf;
-            const bool prev = f < nprev;
-            const int k0 = (f - nprev) * BR_BN;
-            if (f >= f_end || (!prev && k0 >= self_end)) return false;
-            if (prev && table && f - dbase >= 64) {
-                dbase = f;
-                dreg = dbase + lane < nprev ? tiles_b[dbase + lane] : make_int2(0, 0);
-                asm volatile("" : "+v"(dreg.x), "+v"(dreg.y));   // wait here, not at every later use
-            }
-            const int li = (prev && table) ? f - dbase : 0;
-            const int t_tok0 = __builtin_amdgcn_readlane(dreg.x, li), t_nv = __builtin_amdgcn_readlane(dreg.y, li);
-            const int p_nv = it.len0 - f * BR_BN < BR_BN ? it.len0 - f * BR_BN : BR_BN;
-            const int o_nv = self_end - k0 < BR_BN ? self_end - k0 : BR_BN;
-            n_f = f;
-            n_tok0 = prev ? (table ? t_tok0 : it.tok0 + f * BR_BN) : own_tok0 + k0;
-            n_nvalid = prev ? (table ? t_nv : p_nv) : o_nv;
-            wf = f + 1;
-            return true;
-        };
-        bool have = fetch();
-        c_f = n_f; c_tok0 = n_tok0; c_nvalid = n_nvalid;
-        if (have) {
-            int lane_l = lane;
-            asm volatile("" : "+v"(lane_l));
-            issue_tile(L, wave, lane_l, kbase + (long long)c_tok0 * p.sk_t, vbase + (long long)c_tok0 * p.sv_t, sk_bytes, sv_bytes, c_nvalid,
-                       smem_lds);
-        }
-
-        // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.
-        bf16x8 qf[D / 16];
-        {
-            const bool ok = row0 + ln < len_m;
-            const __bf16* qrow = reinterpret_cast<const __bf16*>(p.q) + (long long)b * p.sq_b + (long long)head * p.sq_h +
-                                 (long long)(qtok0 + row0) * p.sq_t;
-            const int qoff = ln * (int)p.sq_t + lh * 8;
-#pragma unroll
-            for (int c = 0; c < D / 16; ++c) {
-                uint4 z = {0u, 0u, 0u, 0u};
-                if (ok) z = ld16(qrow + qoff + c * 16);
-                qf[c] = as_bf16x8(z);
-            }
-        }
-
-        f32x16 o[D / 32];
-#pragma unroll
-        for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o[d][v] = 0.f;
-        float m_run = -INFINITY, l_run = 0.f;
-
-        vm_wait_all();
-        // tell the compiler the Q fragments are in registers now: otherwise it would put its own
-        // "wait for every outstanding load" in front of the first MFMA of each iteration, which would
-        // also wait for the next tile's DMA and undo the overlap
-#pragma unroll
-        for (int c = 0; c < D / 16; ++c) asm volatile("" : "+v"(qf[c]));
-        __syncthreads();
-        int bufi = 0;
-
-        while (have) {
-            // the lane index as a value the compiler cannot trace back: what the rare paths below derive
-            // from it (partial tiles, score partials) is computed there, not kept in registers
-            int lane_l = lane;
-            asm volatile("" : "+v"(lane_l));
-            const bool have_next = fetch();
-            if (have_next)
-                issue_tile(L, wave, lane_l, kbase + (long long)n_tok0 * p.sk_t, vbase + (long long)n_tok0 * p.sv_t, sk_bytes, sv_bytes,
-                           n_nvalid, smem_lds + (bufi ^ 1) * SM::stageBytes);
-            const char* stage = smem + bufi * SM::stageBytes;
-
-            // 32-key halves of the tile this wave needs: limited by the real keys in the tile and, on
-            // the block's own keys, by the diagonal (last row of the wave is row0 + 31).
-            // (the tile quantities are handed to the arithmetic below as per-lane values: with scalar ones
-            // the compiler's code for the four tile variants needs far more registers than there are)
-            int v_nvalid = c_nvalid, v_f = c_f;
-            asm volatile("" : "+v"(v_nvalid), "+v"(v_f));
-            int nkb = (v_nvalid + 31) >> 5;
-            const bool c_self = v_f >= nprev;              // the block's own keys: the causal rule applies
-            const int key0 = (v_f - nprev) * BR_BN;        // then: position of the tile's first key in the block
-            if (c_self) {
-                int vis = row0 + BR_RB - key0;             // keys [0, vis) of the tile are visible to some row
-                int c = vis <= 0 ? 0 : (vis + 31) >> 5;
-                nkb = c < nkb ? c : nkb;
-            }
-            if (!rb_active) nkb = 0;
-            const bool need_mask = (v_nvalid < nkb * 32) || (c_self && key0 + nkb * 32 - 1 > row0);
-            float psum = 0.f;
-            if (nkb == 2 && !need_mask) {
-                compute_tile<2, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, 0, lh, psum);
-            } else if (nkb > 0) {
-                const int lim_causal = c_self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
-                const int lim = v_nvalid < lim_causal ? v_nvalid : lim_causal;
-                if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
-                else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
-                else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
-            }
-            // Score partials: this tile's probability mass (against the running max) for the query block's
-            // last rows, per head - everything the per-document scores need, with no second pass over K.
-            if (emit_scores && nkb > 0 && !c_self && c_f >= first_doc_tile) {
-                const float tot = psum + __shfl_xor(psum, 32);
-                const int ln_l = lane_l & 31;
-                const int r16 = it.start_m + row0 + ln_l - (p.H - p.score_R);
-                if (lane_l < 32 && r16 >= 0 && row0 + ln_l < len_m) {
-                    float2 ms = make_float2(m_run == -INFINITY ? 0.f : m_run, tot);
-                    *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + c_f) * 2) = ms;
-                }
-            }
-
-            if (wave == 0) pf.step();
-            vm_wait_all();
-            __syncthreads();
-            bufi ^= 1;
-            c_f = n_f; c_tok0 = n_tok0; c_nvalid = n_nvalid;
-            have = have_next;
-        }
-
-        // ---- epilogue: lane (ln, lh) holds row row0+ln, dims 32d + 8(v/4) + 4lh + v%4 ----
-        // (the lane index is laundered so that the output addresses are computed here, not hoisted
-        // to the top of the item where they would have to be spilled across the key loop)
-        int lane_e = lane;
-        asm volatile("" : "+v"(lane_e));
-        const float l_tot = l_run + __shfl_xor(l_run, 32);
-        if (it.slot >= 0) {
-            if (row0 + ln < len_m) {
-                const long long slot = ((long long)b * BR_SLOTS_PER_SEQ + it.slot) * ge.NHG + hg;
-                const long long prow = slot * (NW * BR_RB) + wave * BR_RB + ln;
-                float* po = p.part_o + prow * D;
-#pragma unroll
-                for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        f32x4 t = {o[d][4 * q4], o[d][4 * q4 + 1], o[d][4 * q4 + 2], o[d][4 * q4 + 3]};
-                        *reinterpret_cast<f32x4*>(po + d * 32 + 8 * q4 + 4 * lh) = t;
-                    }
-                if (lh == 0) {
-                    p.part_ml[prow * 2] = m_run;
-                    p.part_ml[prow * 2 + 1] = l_tot;
-                }
-            }
-        } else {
-            // the last loop iteration ended with a barrier, so the K/V buffers are free: transpose
-            // through LDS so that every output row is written as full 16-byte pieces
-            __bf16* Es = reinterpret_cast<__bf16*>(smem + wave * SM::eBytesPerWave);
-            const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-            if (rb_active) {
-#pragma unroll
-                for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        f32x4 t = {o[d][4 * q4] * inv, o[d][4 * q4 + 1] * inv, o[d][4 * q4 + 2] * inv,
-                                   o[d][4 * q4 + 3] * inv};
-                        bf16x4 h4 = __builtin_convertvector(t, bf16x4);
-                        *reinterpret_cast<bf16x4*>(Es + ln * SM::eRow + d * 32 + 8 * q4 + 4 * lh) = h4;
-                    }
-                // same wave wrote and reads: LDS operations of one wave complete in order; the fence
-                // keeps the compiler from moving the reads above the writes
-                __threadfence_block();
-                __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h +
-                                (long long)(qtok0 + row0) * p.so_t;
-#pragma unroll
-                for (int i = 0; i < (BR_RB * CPR) / 64; ++i) {
-                    int ch = lane_e + i * 64;
-                    int row = ch / CPR, c8 = ch - row * CPR;
-                    if (row0 + row < len_m) {
-                        uint4 val = ld16(Es + row * SM::eRow + c8 * 8);
-                        *reinterpret_cast<uint4*>(obase + row * (int)p.so_t + c8 * 8) = val;
-                    }
-                }
-            }
-        }
-    }
-};
-
-template <int D, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillParams p) {
-    // one LDS object, so that it starts at LDS address 0 and every DMA target stays below 64 KiB;
-    // the two descriptor mailboxes sit behind the tile stages
-    __shared__ __attribute__((aligned(1024))) char smem[Smem<D>::total(NW) + 2 * sizeof(BrDescMail)];
-    BrDescMail* mail = reinterpret_cast<BrDescMail*>(smem + Smem<D>::total(NW));
-    using PF = Prefill<D, NW>;
-    const int NHG = p.geom.NHG;
-    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
-    int* hdr = const_cast<int*>(p.plan);
-    const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const typename PF::Lane L = PF::make_lane(p, wave, lane);
-    // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
-    for (int i = threadIdx.x * 16; i < Smem<D>::total(NW); i += NW * 64 * 16) *reinterpret_cast<uint4*>(smem + i) = uint4{0u, 0u, 0u, 0u};
-    BrPrefetch pf;
-    pf.init(hdr, &pv, NHG, lane);
-    if (wave == 0) pf.publish(&mail[0]);
-    __syncthreads();
-    for (int cur = 0;; cur ^= 1) {
-        if (uni(mail[cur].valid) == 0) break;
-        BrItem it;
-        {
-            int* w = reinterpret_cast<int*>(&it);
-#pragma unroll
-            for (int i = 0; i < BR_ITEM_WORDS_USED; ++i) w[i] = uni(mail[cur].word[i]);
-        }
-        const int hg = uni(mail[cur].hg);
-        if (wave == 0) pf.draw();
-        PF::run_item(p, pv, it, hg, smem, L, pf);
-        if (wave == 0) pf.publish(&mail[cur ^ 1]);
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) br_leave(hdr);
-}
-
-// Finish: (1) merge the split-KV partials of the query block,
-// out = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m); one workgroup per (query tile, head group, row
-// block); (2) set the rows of padded token slots to zero.
-template <int D>
-__global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int NW) {
-    const BrGeom& ge = p.geom;
-    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
-    constexpr int CPR = D / 4;                    // float4 chunks per row = threads per row
-    constexpr int RPW = 256 / CPR;                // rows one workgroup merges at a time
-    constexpr int SUBS = BR_RB / RPW;             // such row groups per 32-row block
-    const int n_units = pv.hdr[BR_PH_NCOMB] * ge.NHG * NW * SUBS;
-    const int m = p.M - 1;
-    const int rows = NW * BR_RB;
-    const int rr = threadIdx.x / CPR, cc = threadIdx.x % CPR;
-    for (int u = blockIdx.x; u < n_units; u += gridDim.x) {
-        const int subu = u % SUBS;
-        const int wave = (u / SUBS) % NW;
-        const int w = u / (SUBS * NW);
-        const int ci = w / ge.NHG, hg = w - ci * ge.NHG;
-        const BrComb c = pv.comb[ci];
-        const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
-        const int len_m = pv.len[c.b * p.M + m];
-        const int qtok0 = pv.tok[c.b * p.M + m];
-        const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
-        const int rloc = subu * RPW + rr;                            // row inside the 32-row block
-        const int row = c.t0 + sub * BR_RB + rloc;
-        if (row >= len_m) continue;
-        const int head = kvh * ge.G + hsub * ge.Gw + g;
-        const int r = wave * BR_RB + rloc;
-        const long long slot0 = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0) * ge.NHG + hg;
-        const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
-        const float2* ml = reinterpret_cast<const float2*>(p.part_ml) + slot0 * rows + r;
-        const float* po = p.part_o + (slot0 * rows + r) * D + cc * 4;
-        // all loads of up to eight splits are in flight together; a thread owns one float4 of the row
-        float mmax = -INFINITY, l = 0.f;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int s0 = 0; s0 < c.nsplit; s0 += 8) {
-            float2 mls[8];
-            f32x4 ov[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const bool on = s0 + j < c.nsplit;
-                mls[j] = on ? ml[(s0 + j) * sstride] : make_float2(-INFINITY, 0.f);
-                ov[j] = on ? *reinterpret_cast<const f32x4*>(po + (s0 + j) * sstride * D) : f32x4{0.f, 0.f, 0.f, 0.f};
-            }
-            float mnew = mmax;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) mnew = fmaxf(mnew, mls[j].x);
-            const float resc = mmax == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mmax - mnew);
-            l *= resc;
-            acc *= resc;
-            mmax = mnew;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float w8 = mls[j].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mls[j].x - mmax);
-                l += mls[j].y * w8;
-                acc += ov[j] * w8;
-            }
-        }
-        const float inv = l > 0.f ? 1.f / l : 0.f;
-        __bf16* dst = reinterpret_cast<__bf16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
-                      (long long)(qtok0 + row) * p.so_t;
-        bf16x4 h4 = __builtin_convertvector(acc * inv, bf16x4);
-        *reinterpret_cast<bf16x4*>(dst + cc * 4) = h4;
-    }
-    // padded token slots: the kernels never touch them, so give them a defined value (zero)
-    // (a packed layout has none)
-    const int n_pad_work = pv.hdr[BR_PH_PACKED] ? 0 : p.B * p.M * p.Nq;
-    for (int w = blockIdx.x; w < n_pad_work; w += gridDim.x) {
-        const int bm = w / p.Nq, head = w - bm * p.Nq;
-        const int b = bm / p.M, mm = bm - b * p.M;
-        const int st = pv.start[bm], ln = pv.len[bm];
-        const int npad = p.H - ln;
-        constexpr int CP8 = D / 8;
-        __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
-        for (int idx = threadIdx.x; idx < npad * CP8; idx += blockDim.x) {
-            int r = idx / CP8, c8 = idx - r * CP8;
-            int pos = r < st ? r : r + ln;
-            uint4 z = {0u, 0u, 0u, 0u};
-            *reinterpret_cast<uint4*>(obase + (long long)(mm * p.H + pos) * p.so_t + c8 * 8) = z;
-        }
-    }
-}
-
 template <int D, int NW>
 void launch(const BrPrefillParams& p, int grid, hipStream_t stream) {
-    hipLaunchKernelGGL((br_prefill_mfma_kernel<D, NW>), dim3(grid), dim3(NW * 64), 0, stream, p);
+    hipLaunchKernelGGL((br_prefill_mfma_kernel<D, NW, false>), dim3(grid), dim3(NW * 64), 0, stream, p);
 }
 
 }  // namespace

@@ -114,6 +114,24 @@ int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out
                           void* workspace, size_t workspace_bytes, int score_rows, float* score_part,
                           size_t score_part_bytes, void* stream, void* ev_start, void* ev_stop);
 
+/* Bytes of scratch br_prefill_fwd_fp8qk needs: the split-KV partials plus the quantised Q and K.
+ * tokens: length of the token axis summed over the batch (B*M*H for the padded layout, the number of
+ * real tokens for a packed one). */
+size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int64_t tokens);
+
+/* br_prefill_fwd_scores with Q K^T computed in fp8 e4m3 and P V in bf16.  q, k, v, out are bf16 as in
+ * br_prefill_fwd; Q and K are first quantised per (sequence, head) with scale = max|x| / 448 over the
+ * real tokens (x / scale rounded to e4m3), the products run on the fp8 matrix cores and the two scales
+ * are folded into the softmax scale.  D = 128 only.  score_part may be NULL (then score_rows is
+ * ignored).  No reference counterpart: the reference computes Q K^T in the model dtype
+ * (blockrank_std_attention.py:549-620); this is the reduced-precision variant for Qwen2.5-shaped
+ * ranking whose scores must stay within 5e-3 relative of the fp32 result with the same top-10. */
+int br_prefill_fwd_fp8qk(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
+                         int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
+                         const int64_t* v_strides, const int64_t* out_strides, float scale, int64_t tokens,
+                         void* workspace, size_t workspace_bytes, int score_rows, float* score_part,
+                         size_t score_part_bytes, void* stream, void* ev_start, void* ev_stop);
+
 /* Per-document relevance from the partials of br_prefill_fwd_scores: compute_auxiliary_attention_loss(
  * answer_ids=None, return_logits=True) (src/blockrank/losses.py:37-78).
  *   rows: (B, R) int32 indices 0..score_rows-1 into the last score_rows positions of the query block

@@ -99,3 +99,29 @@ def test_topk_is_stable_descending():
     s = np.array([[0.1, 0.9, 0.9, 0.3], [3.0, 1.0, 2.0, 2.0]])
     assert orc.topk_indices(s, 3).tolist() == [[1, 2, 3], [0, 2, 3]]
     assert orc.topk_indices(s, 10).shape == (2, 4)
+
+
+def test_fp8_quantiser_pins():
+    """quantize_fp8_e4m3: representable values survive, the per-head maximum is exact, the relative
+    round-trip error of normal values is at most 2^-4, padded positions come back as zero."""
+    import torch
+    from oracle import blockrank_oracle as orc
+    valid = torch.ones(1, 2, 4, dtype=torch.bool)
+    valid[0, 0, 0] = False
+    # e4m3 values (scaled so that the maximum maps to 448): 448, 416, 1.0, 0.875, 2^-6 (smallest normal), 0
+    vals = torch.tensor([0.0, 448.0, -416.0, 1.0, 0.875, 2.0 ** -6, 3.5, -240.0])
+    x = torch.zeros(1, 1, 8, 4)
+    x[0, 0, :, 0] = vals * 0.37                       # any common factor must cancel
+    x[0, 0, 0, :] = 1e6                               # padded position: must not set the scale
+    got = orc.quantize_fp8_e4m3(x, valid)
+    assert torch.equal(got[0, 0, 0], torch.zeros(4))
+    torch.testing.assert_close(got[0, 0, 1:, 0], x[0, 0, 1:, 0], rtol=1e-6, atol=0)
+    g = torch.Generator().manual_seed(0)
+    y = torch.randn(2, 3, 8, 16, generator=g)
+    v2 = torch.ones(2, 2, 4, dtype=torch.bool)
+    r = orc.quantize_fp8_e4m3(y, v2)
+    amax = y.abs().amax(dim=(2, 3))
+    torch.testing.assert_close(r.abs().amax(dim=(2, 3)), amax, rtol=1e-6, atol=0)
+    normal = y.abs() >= (amax / 448.0 * 2.0 ** -6)[:, :, None, None]
+    rel = ((r - y).abs() / y.abs())[normal]
+    assert rel.max().item() <= 2.0 ** -4 + 1e-6
