@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BlockRank attention + per-document score path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5shape|cfg1] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5shape|cfg1] [--qk-fp8] [--no-cpu-baseline]
 
 A step is one pass of the hot path over one batch already resident in HBM: the attention hook
 (block-sparse prefill attention of one layer, query/key/value as a Mistral layer hands them over)
@@ -201,6 +201,8 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
+    ap.add_argument("--qk-fp8", action="store_true",
+                    help="compute Q K^T in fp8 e4m3 (bf16 workloads with head dim 128; includes the quantisation pass)")
     ap.add_argument("--padded", action="store_true",
                     help="cfg3: feed the reference's padded (B, M, H) batch instead of the packed one")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -244,7 +246,8 @@ def main():
     plan_ms = (time.perf_counter() - t0) * 1e3
 
     def step(events=None):
-        out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events)
+        out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events,
+                                                      qk_fp8=args.qk_fp8)
         scores = handle.doc_scores_window(rows16, temperature=0.05) if handle is not None else None
         return out, scores
 
@@ -317,7 +320,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if dtype == torch.bfloat16 else "f32",
+        "dtype": ("fp8 e4m3 (Q K^T) + bf16 (P V)" if args.qk_fp8 else "bf16") if dtype == torch.bfloat16 else "f32",
         "data": "synthetic",
         "config": {"workload": wl["desc"], "name": args.workload, "batch": layout.B, "blocks": layout.M, "block_len": layout.H,
                    "valid_tokens": layout.valid_tokens, "unmasked_pairs": pairs_n, "launch": "graph" if graph_ms is not None and graph_ms < ms_per_step else "eager"},

@@ -280,17 +280,32 @@ struct Prefill {
                                              int sv_bytes, int nvalid, unsigned stage_lds) {
         // rows past a partial tile's real keys are not fetched: the LDS rows keep older (finite) data,
         // which the kernel masks (K) or multiplies by exact zeros (V)
-        const bool full = nvalid == BR_BN;
+        if (nvalid == BR_BN) {
+            // whole tile: straight-line issue, no per-piece predicate
+#pragma unroll
+            for (int j = 0; j < JKK; ++j) {
+                const int q = wave + NW * j;
+                if (NIK % NW == 0 || q < NIK) {
+                    if (UNIFORM_STEP) dma16(kt + j * STEP_ROWSK * sk_bytes, L.koff[0], stage_lds + q * 1024);
+                    else dma16(kt, L.koff[j], stage_lds + q * 1024);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < JK; ++j) {
+                const int q = wave + NW * j;
+                if (NI % NW == 0 || q < NI) {
+                    if (UNIFORM_STEP) dma16(vt + j * STEP_ROWS * sv_bytes, L.voff[0], stage_lds + SM::kBytes + q * 1024);
+                    else dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < JKK; ++j) {
             const int q = wave + NW * j;
             if (NIK % NW == 0 || q < NIK) {
-                bool on = true;
-                if (!full) {
-                    const int prow = (q * 64 + lane_l) / CPRK;
-                    on = ((prow & 32) | swap23(prow & 31)) < nvalid;           // K row of this piece
-                }
-                if (on) {
+                const int prow = (q * 64 + lane_l) / CPRK;
+                if (((prow & 32) | swap23(prow & 31)) < nvalid) {                  // K row of this piece
                     if (UNIFORM_STEP) dma16(kt + j * STEP_ROWSK * sk_bytes, L.koff[0], stage_lds + q * 1024);
                     else dma16(kt, L.koff[j], stage_lds + q * 1024);
                 }
@@ -300,9 +315,7 @@ struct Prefill {
         for (int j = 0; j < JK; ++j) {
             const int q = wave + NW * j;
             if (NI % NW == 0 || q < NI) {
-                bool on = true;
-                if (!full) on = (q * 64 + lane_l) / CPR < nvalid;              // V row of this piece
-                if (on) {
+                if ((q * 64 + lane_l) / CPR < nvalid) {                            // V row of this piece
                     if (UNIFORM_STEP) dma16(vt + j * STEP_ROWS * sv_bytes, L.voff[0], stage_lds + SM::kBytes + q * 1024);
                     else dma16(vt, L.voff[j], stage_lds + SM::kBytes + q * 1024);
                 }
@@ -461,7 +474,37 @@ struct Prefill {
         int wf = it.f_lo;                                  // next tile of the walk
         int dbase = it.f_lo;
         int2 dreg = make_int2(0, 0);
-        if (table && dbase + lane < nprev) dreg = tiles_b[dbase + lane];
+        if (table) {
+            if (dbase + lane < nprev) dreg = tiles_b[dbase + lane];
+            // wait for the table here: a wait placed later would also cover the Q loads issued below
+            asm volatile("" : "+v"(dreg.x), "+v"(dreg.y));
+        }
+        // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.  Requested
+        // early (they come from HBM; only the tile table's load, which the walk needs first, goes before them):
+        // the rest of the set-up runs under their latency.
+        Frag qf[D / 16];
+        {
+            const char* qrow = reinterpret_cast<const char*>(p.q) +
+                               ((unsigned long long)p.sq_b * (unsigned)b + (unsigned long long)p.sq_h * (unsigned)head +
+                                (unsigned long long)p.sq_t * (unsigned)(qtok0 + row0)) * ESZ;
+            // rows past the block's end load its last row instead (no per-lane branches around the loads):
+            // what such rows compute is never stored
+            const int last = len_m - 1 - row0;
+            const int qoff = ((ln < last ? ln : last) * (int)p.sq_t + lh * 8) * ESZ;
+            if (rb_active) {
+#pragma unroll
+                for (int c = 0; c < D / 16; ++c) {
+                    if constexpr (F8) qf[c] = *reinterpret_cast<const k8x8*>(qrow + qoff + c * 16);
+                    else qf[c] = as_bf16x8(ld16(qrow + qoff + c * 32));
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < D / 16; ++c) {
+                    if constexpr (F8) qf[c] = 0;
+                    else qf[c] = as_bf16x8(uint4{0u, 0u, 0u, 0u});
+                }
+            }
+        }
         // tile state: index in the walk (earlier-block tiles come first, f < nprev; then the block's
         // own tiles), first token, real keys
         int c_f = 0, c_tok0 = 0, c_nvalid = 0;
@@ -493,27 +536,6 @@ struct Prefill {
             asm volatile("" : "+v"(lane_l));
             issue_tile(L, wave, lane_l, kbase + (long long)c_tok0 * sk_bytes, vbase + (long long)c_tok0 * sv_bytes, sk_bytes, sv_bytes, c_nvalid,
                        smem_lds);
-        }
-
-        // Q^T fragments: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 for every chunk c.
-        Frag qf[D / 16];
-        {
-            const bool ok = row0 + ln < len_m;
-            const char* qrow = reinterpret_cast<const char*>(p.q) +
-                               ((long long)b * p.sq_b + (long long)head * p.sq_h + (long long)(qtok0 + row0) * p.sq_t) * ESZ;
-            const int qoff = (ln * (int)p.sq_t + lh * 8) * ESZ;
-#pragma unroll
-            for (int c = 0; c < D / 16; ++c) {
-                if constexpr (F8) {
-                    k8x8 z = 0;
-                    if (ok) z = *reinterpret_cast<const k8x8*>(qrow + qoff + c * 16);
-                    qf[c] = z;
-                } else {
-                    uint4 z = {0u, 0u, 0u, 0u};
-                    if (ok) z = ld16(qrow + qoff + c * 32);
-                    qf[c] = as_bf16x8(z);
-                }
-            }
         }
 
         f32x16 o[D / 32];
@@ -616,7 +638,7 @@ struct Prefill {
             // the last loop iteration ended with a barrier, so the K/V buffers are free: transpose
             // through LDS so that every output row is written as full 16-byte pieces
             __bf16* Es = reinterpret_cast<__bf16*>(smem + wave * SM::eBytesPerWave);
-            const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+            const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;
             if (rb_active) {
 #pragma unroll
                 for (int d = 0; d < D / 32; ++d)
@@ -630,16 +652,26 @@ struct Prefill {
                 // same wave wrote and reads: LDS operations of one wave complete in order; the fence
                 // keeps the compiler from moving the reads above the writes
                 __threadfence_block();
-                __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h +
-                                (long long)(qtok0 + row0) * p.so_t;
+                // lane -> (row rsub of each group of RPI rows, 16-byte piece c8); all reads first, then
+                // the stores, whose addresses differ by a uniform step
+                constexpr int RPI = 64 / CPR, NIT = BR_RB / RPI;
+                const unsigned le = (unsigned)lane_e;
+                const unsigned rsub = le / CPR, c8 = le % CPR;
+                uint4 vals[NIT];
 #pragma unroll
-                for (int i = 0; i < (BR_RB * CPR) / 64; ++i) {
-                    int ch = lane_e + i * 64;
-                    int row = ch / CPR, c8 = ch - row * CPR;
-                    if (row0 + row < len_m) {
-                        uint4 val = ld16(Es + row * SM::eRow + c8 * 8);
-                        *reinterpret_cast<uint4*>(obase + row * (int)p.so_t + c8 * 8) = val;
-                    }
+                for (int i = 0; i < NIT; ++i) vals[i] = ld16(Es + (rsub + i * RPI) * SM::eRow + c8 * 8);
+                const unsigned long long row_first = (unsigned)(qtok0 + row0);
+                char* optr = reinterpret_cast<char*>(p.out) +
+                             2 * ((unsigned long long)p.so_b * (unsigned)b + (unsigned long long)p.so_h * (unsigned)head +
+                                  (unsigned long long)p.so_t * (row_first + rsub) + c8 * 8);
+                const long long stepb = 2LL * RPI * p.so_t;
+                if (row0 + BR_RB <= len_m) {
+#pragma unroll
+                    for (int i = 0; i < NIT; ++i) *reinterpret_cast<uint4*>(optr + i * stepb) = vals[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NIT; ++i)
+                        if (row0 + (int)rsub + i * RPI < len_m) *reinterpret_cast<uint4*>(optr + i * stepb) = vals[i];
                 }
             }
         }
