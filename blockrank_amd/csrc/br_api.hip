@@ -107,7 +107,7 @@ int check_strides(const char* name, const int64_t* s, int dtype) {
     return BR_OK;
 }
 
-size_t slots_total(int B, const BrGeom& g) { return (size_t)B * BR_SLOTS_PER_SEQ * g.NHG; }
+size_t slots_total(int B, const BrGeom& g, int slots = BR_SLOTS_PER_SEQ) { return (size_t)B * slots * g.NHG; }
 
 }  // namespace
 
@@ -172,6 +172,14 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     return rows * (size_t)(D + 2) * sizeof(float);
 }
 
+size_t br_prefill_workspace_bytes_fused(int B, int M, int Nq, int Nkv, int D) {
+    BrGeom g;
+    int nw;
+    if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || D <= 0 || M <= 0) return 0;
+    size_t rows = slots_total(B, g, br_slots_view1(M)) * (size_t)nw * BR_RB;
+    return rows * (size_t)(D + 2) * sizeof(float);
+}
+
 size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows) {
     if (B <= 0 || Nq <= 0 || M < 3 || H <= 0 || score_rows <= 0) return 0;
     return (size_t)B * Nq * score_rows * br_plan_tps(M, H) * 2 * sizeof(float);
@@ -220,7 +228,16 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
 
     BrPrefillParams p;
     p.q = q; p.k = k; p.v = v; p.out = out; p.plan = plan;
-    const size_t rows = slots_total(B, g) * (size_t)nw * BR_RB;
+    // The fused path (bf16: sequences of short blocks go to the resident kernel, the query block's rows are
+    // computed with each block) needs M-dependent room for partials.  It is opt-in for now - with
+    // BLOCKRANK_AMD_RESIDENT=1, and only when the caller's workspace has that room: on the measured
+    // workloads it does not beat the streaming kernel yet.
+    const char* res_env = getenv("BLOCKRANK_AMD_RESIDENT");
+    const bool fused = dtype == BR_DTYPE_BF16 && fp8_tokens == 0 && (D == 64 || D == 128) && res_env && atoi(res_env) != 0 &&
+                       workspace_bytes >= br_prefill_workspace_bytes_fused(B, M, Nq, Nkv, D);
+    p.queue_view = fused ? 1 : 0;
+    p.slots = fused ? br_slots_view1(M) : BR_SLOTS_PER_SEQ;
+    const size_t rows = slots_total(B, g, p.slots) * (size_t)nw * BR_RB;
     p.part_o = static_cast<float*>(workspace);
     p.part_ml = p.part_o + rows * D;
     p.sq_b = q_strides[0]; p.sq_h = q_strides[1]; p.sq_t = q_strides[2];

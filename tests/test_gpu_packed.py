@@ -60,7 +60,7 @@ def test_plan_from_lengths_equals_plan_from_mask():
     a = br.BlockMask(lay.valid.to(DEV), torch.bfloat16)
     b = br.BlockMask.from_lengths(torch.as_tensor(lay.lengths, dtype=torch.int32, device=DEV), H=lay.H, packed=False)
     pa, pb = a.plan(8, 2), b.plan(8, 2)
-    n = 64 + 3 * lay.B * lay.M                      # header, block starts, lengths and token table
+    n = 96 + 3 * lay.B * lay.M                      # header, block starts, lengths and token table
     assert torch.equal(pa[:n], pb[:n])
     assert torch.equal(br.blockrank_attention(q, k, v, a, 0.125), br.blockrank_attention(q, k, v, b, 0.125))
     assert torch.equal(b.dense(torch.bfloat16), a.dense(torch.bfloat16))
