@@ -244,6 +244,13 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     p.sk_b = k_strides[0]; p.sk_h = k_strides[1]; p.sk_t = k_strides[2];
     p.sv_b = v_strides[0]; p.sv_h = v_strides[1]; p.sv_t = v_strides[2];
     p.so_b = out_strides[0]; p.so_h = out_strides[1]; p.so_t = out_strides[2];
+    for (const int64_t* st : {q_strides, k_strides, v_strides, out_strides})
+        for (int i = 0; i < 3; ++i)
+            if (st[i] < 0 || st[i] >= (int64_t(1) << 31)) return fail(BR_ERR_ARG, "strides must be below 2^31 elements (got %lld)", (long long)st[i]);
+    p.q32_b = (unsigned)q_strides[0]; p.q32_h = (unsigned)q_strides[1]; p.q32_t = (unsigned)q_strides[2];
+    p.k32_b = (unsigned)k_strides[0]; p.k32_h = (unsigned)k_strides[1]; p.k32_t = (unsigned)k_strides[2];
+    p.v32_b = (unsigned)v_strides[0]; p.v32_h = (unsigned)v_strides[1]; p.v32_t = (unsigned)v_strides[2];
+    p.o32_b = (unsigned)out_strides[0]; p.o32_h = (unsigned)out_strides[1]; p.o32_t = (unsigned)out_strides[2];
     p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H;
     p.geom = g;
     p.scale_log2 = scale * 1.4426950408889634f;
@@ -274,6 +281,10 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         p.q = q8; p.k = k8;
         p.sq_b = q8_b; p.sq_h = q8_h; p.sq_t = D;
         p.sk_b = k8_b; p.sk_h = k8_h; p.sk_t = D;
+        if (q8_b >= (1LL << 31) || q8_h >= (1LL << 31) || k8_b >= (1LL << 31) || k8_h >= (1LL << 31))
+            return fail(BR_ERR_ARG, "fp8 staging strides must be below 2^31 elements");
+        p.q32_b = (unsigned)q8_b; p.q32_h = (unsigned)q8_h; p.q32_t = (unsigned)D;
+        p.k32_b = (unsigned)k8_b; p.k32_h = (unsigned)k8_h; p.k32_t = (unsigned)D;
         p.qk_scales = scales;
         lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1);
     } else {

@@ -263,6 +263,9 @@ struct BrPrefillParams {
     long long sk_b, sk_h, sk_t;
     long long sv_b, sv_h, sv_t;
     long long so_b, so_h, so_t;
+    // the same strides as 32-bit values (the entry points reject strides of 2^31 elements or more): the
+    // MFMA kernels use these - half the registers, and 32 x 32 -> 64 bit multiplies for the addresses
+    unsigned q32_b, q32_h, q32_t, k32_b, k32_h, k32_t, v32_b, v32_h, v32_t, o32_b, o32_h, o32_t;
     int B, Nq, Nkv, M, H;
     BrGeom geom;
     float scale_log2;  // softmax scale * log2(e)

@@ -257,13 +257,13 @@ struct Prefill {
             const int slot = (wave + NW * j) * 64 + lane;
             const int prow = slot / CPRK, cp = slot - prow * CPRK;
             const int kkey = (prow & 32) | swap23(prow & 31);
-            L.koff[j] = kkey * (int)p.sk_t * ESZ + ((cp ^ (prow & (CPRK < 8 ? CPRK - 1 : 7))) << 4);
+            L.koff[j] = kkey * (int)p.k32_t * ESZ + ((cp ^ (prow & (CPRK < 8 ? CPRK - 1 : 7))) << 4);
         }
 #pragma unroll
         for (int j = 0; j < JO; ++j) {
             const int slot = (wave + NW * j) * 64 + lane;
             const int prow = slot / CPR, cp = slot - prow * CPR;
-            L.voff[j] = prow * (int)p.sv_t * 2 + ((cp ^ ((prow & 3) << 1)) << 4);
+            L.voff[j] = prow * (int)p.v32_t * 2 + ((cp ^ ((prow & 3) << 1)) << 4);
         }
         const int ln = lane & 31, lh = lane >> 5;
         if (F8) L.krd = ln * SM::rowKB + (((ln & (CPRK < 8 ? CPRK - 1 : 7))) << 4) + lh * 8;   // 8 bytes: dims 16c + 8lh .. +7
@@ -451,10 +451,10 @@ struct Prefill {
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
         const int qtok0 = it.tok_m;                        // token index of the block's first real token
         const unsigned smem_lds = lds_addr_of(smem);
-        const int sk_bytes = (int)p.sk_t * ESZ, sv_bytes = (int)p.sv_t * 2;
+        const int sk_bytes = (int)p.k32_t * ESZ, sv_bytes = (int)p.v32_t * 2;
 
-        const char* kbase = reinterpret_cast<const char*>(p.k) + ((long long)b * p.sk_b + (long long)kvh * p.sk_h) * ESZ;
-        const char* vbase = reinterpret_cast<const char*>(p.v) + ((long long)b * p.sv_b + (long long)kvh * p.sv_h) * 2;
+        const char* kbase = reinterpret_cast<const char*>(p.k) + ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh) * ESZ;
+        const char* vbase = reinterpret_cast<const char*>(p.v) + ((unsigned long long)p.v32_b * (unsigned)b + (unsigned long long)p.v32_h * (unsigned)kvh) * 2;
         // fp8 Q/K: the two dequantisation scales of this (sequence, head) pair go into the softmax scale
         float sc2 = p.scale_log2;
         if constexpr (F8) {
@@ -490,12 +490,12 @@ struct Prefill {
         Frag qf[D / 16];
         {
             const char* qrow = reinterpret_cast<const char*>(p.q) +
-                               ((unsigned long long)p.sq_b * (unsigned)b + (unsigned long long)p.sq_h * (unsigned)head +
-                                (unsigned long long)p.sq_t * (unsigned)(qtok0 + row0)) * ESZ;
+                               ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)head +
+                                (unsigned long long)p.q32_t * (unsigned)(qtok0 + row0)) * ESZ;
             // rows past the block's end load its last row instead (no per-lane branches around the loads):
             // what such rows compute is never stored
             const int last = len_m - 1 - row0;
-            const int qoff = ((ln < last ? ln : last) * (int)p.sq_t + lh * 8) * ESZ;
+            const int qoff = ((ln < last ? ln : last) * (int)p.q32_t + lh * 8) * ESZ;
             if (rb_active) {
 #pragma unroll
                 for (int c = 0; c < D / 16; ++c) {
@@ -667,9 +667,9 @@ struct Prefill {
                 for (int i = 0; i < NIT; ++i) vals[i] = ld16(Es + (rsub + i * RPI) * SM::eRow + c8 * 8);
                 const unsigned long long row_first = (unsigned)(qtok0 + row0);
                 char* optr = reinterpret_cast<char*>(p.out) +
-                             2 * ((unsigned long long)p.so_b * (unsigned)b + (unsigned long long)p.so_h * (unsigned)head +
-                                  (unsigned long long)p.so_t * (row_first + rsub) + c8 * 8);
-                const long long stepb = 2LL * RPI * p.so_t;
+                             2 * ((unsigned long long)p.o32_b * (unsigned)b + (unsigned long long)p.o32_h * (unsigned)head +
+                                  (unsigned long long)p.o32_t * (row_first + rsub) + c8 * 8);
+                const long long stepb = 2LL * RPI * p.o32_t;
                 if (row0 + BR_RB <= len_m) {
 #pragma unroll
                     for (int i = 0; i < NIT; ++i) *reinterpret_cast<uint4*>(optr + i * stepb) = vals[i];
@@ -748,10 +748,10 @@ struct Resident {
                                                   typename PF::Frag (&qf)[D / 16]) {
         const int ln = lane & 31, lh = lane >> 5;
         const char* qrow = reinterpret_cast<const char*>(p.q) +
-                           ((unsigned long long)p.sq_b * (unsigned)b + (unsigned long long)p.sq_h * (unsigned)head +
-                            (unsigned long long)p.sq_t * (unsigned)(q_tok + row0)) * 2;
+                           ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)head +
+                            (unsigned long long)p.q32_t * (unsigned)(q_tok + row0)) * 2;
         const int last = q_len - 1 - row0;       // rows past the block's end load its last row; they are never stored
-        const int qoff = ((ln < last ? ln : last) * (int)p.sq_t + lh * 8) * 2;
+        const int qoff = ((ln < last ? ln : last) * (int)p.q32_t + lh * 8) * 2;
 #pragma unroll
         for (int c = 0; c < D / 16; ++c) qf[c] = as_bf16x8(ld16(qrow + qoff + c * 32));
     }
@@ -845,8 +845,8 @@ struct Resident {
         // gives every lane whole 16-byte pieces: dims 32d + 16e + 8lh + 0..7 (e = 0, 1).
         const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;
         char* orow = reinterpret_cast<char*>(p.out) +
-                     2 * ((unsigned long long)p.so_b * (unsigned)b + (unsigned long long)p.so_h * (unsigned)head +
-                          (unsigned long long)p.so_t * (unsigned)(q_tok + row0 + ln_e) + lh_e * 8);
+                     2 * ((unsigned long long)p.o32_b * (unsigned)b + (unsigned long long)p.o32_h * (unsigned)head +
+                          (unsigned long long)p.o32_t * (unsigned)(q_tok + row0 + ln_e) + lh_e * 8);
 #pragma unroll
         for (int d = 0; d < D / 32; ++d)
 #pragma unroll
@@ -882,7 +882,7 @@ __global__ __launch_bounds__(512, 1) void br_prefill_resident_kernel(BrPrefillPa
     const int n_tickets = hdr[BR_PH_NRES] * NHG;
     const int res_off = hdr[BR_PH_RES_OFF];
     const unsigned smem_lds = lds_addr_of(rsmem);
-    const int sk_bytes = (int)p.sk_t * 2, sv_bytes = (int)p.sv_t * 2;
+    const int sk_bytes = (int)p.k32_t * 2, sv_bytes = (int)p.v32_t * 2;
     const int T = ge.tpb * BR_RB;
     const float inv_gw = 1.0f / (float)ge.Gw;
     // the first ticket of a workgroup is its index; later ones come from the counter
@@ -909,8 +909,8 @@ __global__ __launch_bounds__(512, 1) void br_prefill_resident_kernel(BrPrefillPa
         const int q_len = it.t0, q_tok = it.f_lo;               // the query block's span (see the plan)
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int n0 = it.nprev, n1 = (it.len_m + BR_BN - 1) / BR_BN;
-        const char* kbase = reinterpret_cast<const char*>(p.k) + ((unsigned long long)p.sk_b * (unsigned)b + (unsigned long long)p.sk_h * (unsigned)kvh) * 2;
-        const char* vbase = reinterpret_cast<const char*>(p.v) + ((unsigned long long)p.sv_b * (unsigned)b + (unsigned long long)p.sv_h * (unsigned)kvh) * 2;
+        const char* kbase = reinterpret_cast<const char*>(p.k) + ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh) * 2;
+        const char* vbase = reinterpret_cast<const char*>(p.v) + ((unsigned long long)p.v32_b * (unsigned)b + (unsigned long long)p.v32_h * (unsigned)kvh) * 2;
         {
             int lane_l = lane;
             asm volatile("" : "+v"(lane_l));
