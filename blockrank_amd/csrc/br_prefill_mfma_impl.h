@@ -702,14 +702,17 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     if (wave == 0) pf.publish(&mail[0]);
     __syncthreads();
     for (int cur = 0;; cur ^= 1) {
-        if (uni(mail[cur].valid) == 0) break;
+        // one LDS read per lane (lane i: word i of the mailbox), then the words are taken from the lanes
+        const int mw = reinterpret_cast<const int*>(&mail[cur])[lane < BR_ITEM_INTS + 2 ? lane : 0];
+#define BR_W(i) __builtin_amdgcn_readlane(mw, i)
+        if (BR_W(BR_ITEM_INTS + 1) == 0) break;     // .valid
         BrItem it;
-        {
-            int* w = reinterpret_cast<int*>(&it);
-#pragma unroll
-            for (int i = 0; i < BR_ITEM_WORDS_USED; ++i) w[i] = uni(mail[cur].word[i]);
-        }
-        const int hg = uni(mail[cur].hg);
+        it.b = BR_W(0); it.m = BR_W(1); it.t0 = BR_W(2); it.f_lo = BR_W(3); it.nprev = BR_W(4); it.ntiles = BR_W(5); it.slot = BR_W(6);
+        it.pe = BR_W(7); it.len_m = BR_W(8); it.start_m = BR_W(9); it.len0 = BR_W(10); it.start0 = BR_W(11); it.tok_m = BR_W(12);
+        it.tok0 = BR_W(13);
+        it.pad[0] = it.pad[1] = 0;
+        const int hg = BR_W(BR_ITEM_INTS);          // .hg
+#undef BR_W
         if (wave == 0) pf.draw();
         PF::run_item(p, pv, it, hg, smem, L, pf);
         if (wave == 0) pf.publish(&mail[cur ^ 1]);
