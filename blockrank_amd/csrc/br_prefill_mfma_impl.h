@@ -694,6 +694,13 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
     const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    {   // nothing queued at all (every sequence went to the resident kernel): leave at once
+        const int c = lane < BR_NQUEUES ? hdr[(p.queue_view == 1 ? BR_PH_QCOUNT2 : BR_PH_QCOUNT) + lane] : 0;
+        if (__builtin_amdgcn_ballot_w64(c > 0) == 0) {
+            if (threadIdx.x == 0) br_leave(hdr);
+            return;
+        }
+    }
     const typename PF::Lane L = PF::make_lane(p, wave, lane);
     // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
     for (int i = threadIdx.x * 16; i < Smem<D, F8>::total(NW); i += NW * 64 * 16) *reinterpret_cast<uint4*>(smem + i) = uint4{0u, 0u, 0u, 0u};
@@ -879,10 +886,14 @@ __global__ __launch_bounds__(512, 1) void br_prefill_resident_kernel(BrPrefillPa
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
     const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int n_tickets = hdr[BR_PH_NRES] * NHG;
+    if ((int)blockIdx.x >= n_tickets) {       // no item for this workgroup (none at all when no sequence is fused)
+        if (threadIdx.x == 0) br_leave_resident(hdr);
+        return;
+    }
     const typename PF::Lane L = PF::make_lane(p, wave, lane);
     // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
     for (int i = threadIdx.x * 16; i < R::kStageBytes; i += 512 * 16) *reinterpret_cast<uint4*>(rsmem + i) = uint4{0u, 0u, 0u, 0u};
-    const int n_tickets = hdr[BR_PH_NRES] * NHG;
     const int res_off = hdr[BR_PH_RES_OFF];
     const unsigned smem_lds = lds_addr_of(rsmem);
     const int sk_bytes = (int)p.k32_t * 2, sv_bytes = (int)p.v32_t * 2;
