@@ -43,6 +43,10 @@ def test_pure_host_entry_points():
     assert lib.br_plan_ints(0, 22, 160, 32, 8) == 0
     assert lib.br_prefill_workspace_bytes(4, 32, 8, 128) == 4 * 32 * 8 * 128 * 130 * 4
     assert lib.br_doc_scores_workspace_bytes(4, 32, 22, 2) == 4 * 32 * 2 * 20 * 2 * 4
+    # the fused path keeps one partial slot per (query tile, block): 2 * M slots, never fewer than the 32 of the split path
+    assert lib.br_prefill_workspace_bytes_fused(4, 22, 32, 8, 128) == 4 * 44 * 8 * 128 * 130 * 4
+    assert lib.br_prefill_workspace_bytes_fused(4, 5, 32, 8, 128) == lib.br_prefill_workspace_bytes(4, 32, 8, 128)
+    assert lib.br_prefill_fp8qk_workspace_bytes(4, 32, 8, 128, 4 * 3520) > lib.br_prefill_workspace_bytes(4, 32, 8, 128)
     # argument errors come back as codes with a message, before anything touches a device
     rc = lib.br_prefill_fwd(None, None, None, None, None, 1, 4, 2, 3, 8, 96, None, None, None, None, 1.0, 1, None, 0, None)
     assert rc == _lib.BR_ERR_ARG and b"head dim" in lib.br_last_error()
@@ -127,3 +131,11 @@ def test_tensor_path_of_loss_matches_oracle_on_cpu():
     got = br.compute_auxiliary_attention_loss(s, labels, valid, answer_ids=None, return_logits=True)
     want = orc.doc_scores_from_logits(s.numpy(), labels.numpy(), valid.numpy(), 0.05)
     np.testing.assert_allclose(got.numpy(), want, rtol=1e-10)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
