@@ -80,6 +80,28 @@ __device__ inline unsigned lds_addr_of(const void* p) {
     return (unsigned)(size_t)(__attribute__((address_space(3))) const void*)p;
 }
 
+// Zero the output rows of a block's padded token slots (padded layout: the block's H slots start at token
+// slot0; its real tokens are [start, start + len)), for heads head0 .. head0 + nheads - 1.  Called by
+// all nthreads threads of a workgroup; plain 16-byte stores, nothing waits for them.
+template <int D>
+__device__ inline void zero_padded_rows(const BrPrefillParams& p, int b, int head0, int nheads, int slot0, int start, int len, int tid,
+                                        int nthreads) {
+    constexpr int CP8 = D / 8;                    // 16-byte pieces per row (a power of two)
+    const int npad = p.H - len;
+    if (npad <= 0) return;
+    const uint4 z = {0u, 0u, 0u, 0u};
+    for (int g = 0; g < nheads; ++g) {
+        char* obase = reinterpret_cast<char*>(p.out) +
+                      2 * ((unsigned long long)p.o32_b * (unsigned)b + (unsigned long long)p.o32_h * (unsigned)(head0 + g) +
+                           (unsigned long long)p.o32_t * (unsigned)slot0);
+        for (int idx = tid; idx < npad * CP8; idx += nthreads) {
+            const int r = idx / CP8, c8 = idx - r * CP8;
+            const int pos = r < start ? r : r + len;
+            *reinterpret_cast<uint4*>(obase + 2 * ((long long)pos * p.o32_t + c8 * 8)) = z;
+        }
+    }
+}
+
 // Exchange bits 2 and 3.  MFMA row r of a 32-key half tile carries key swap23(r): with the 32x32
 // accumulator layout (lane = column + 32*h; register v is row 8*(v/4) + 4*h + v%4) registers
 // 8*jp .. 8*jp+7 of lane half h then hold keys 16*jp + 8*h + 0..7, which is the B-operand layout of
@@ -436,7 +458,7 @@ struct Prefill {
     }
 
     static __device__ void run_item(const BrPrefillParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem,
-                                    const Lane& L, BrPrefetch& pf) {
+                                    const Lane& L, BrPrefetch& pf, bool padded_layout) {
         const int tid = threadIdx.x;
         const int wave = uni(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
         const BrGeom& ge = p.geom;
@@ -680,6 +702,11 @@ struct Prefill {
                 }
             }
         }
+        // A document's padded slots get zeros from the item that holds its first query tile (one such item per
+        // document and head group; a packed layout has no padded slots).  The prefix's and the query block's
+        // are left to the finish kernel: their items are the ones the others wait for.
+        if (it.t0 == 0 && m > 0 && m < p.M - 1 && padded_layout)
+            zero_padded_rows<D>(p, b, kvh * ge.G + hsub * ge.Gw, ge.Gw, it.tok_m - it.start_m, it.start_m, len_m, tid, NW * 64);
     }
 };
 
@@ -704,6 +731,7 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     const typename PF::Lane L = PF::make_lane(p, wave, lane);
     // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
     for (int i = threadIdx.x * 16; i < Smem<D, F8>::total(NW); i += NW * 64 * 16) *reinterpret_cast<uint4*>(smem + i) = uint4{0u, 0u, 0u, 0u};
+    const bool padded_layout = uni(hdr[BR_PH_PACKED]) == 0;
     BrPrefetch pf;
     pf.init(hdr, &pv, NHG, lane, p.queue_view);
     if (wave == 0) pf.publish(&mail[0]);
@@ -721,7 +749,7 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
         const int hg = BR_W(BR_ITEM_INTS);          // .hg
 #undef BR_W
         if (wave == 0) pf.draw();
-        PF::run_item(p, pv, it, hg, smem, L, pf);
+        PF::run_item(p, pv, it, hg, smem, L, pf, padded_layout);
         if (wave == 0) pf.publish(&mail[cur ^ 1]);
         __syncthreads();
     }
@@ -1071,13 +1099,17 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
         bf16x4 h4 = __builtin_convertvector(acc * inv, bf16x4);
         *reinterpret_cast<bf16x4*>(dst + cc * 4) = h4;
     }
-    // padded token slots: the kernels never touch them, so give them a defined value (zero)
-    // (a packed layout has none)
+    // Padded token slots: no kernel computes them, so give them a defined value (zero).  The prefill kernels
+    // streaming kernel does that for the documents it has items for; what is left here are the prefix and
+    // the query block, documents with no real token at all, and the blocks of the fused sequences, which the
+    // resident kernel computes (a packed layout has no padded slots).
+    const int* fused = p.plan + br_plan_off_fused(p.B, p.M, p.H, ge.tpb * BR_RB);
     const int n_pad_work = pv.hdr[BR_PH_PACKED] ? 0 : p.B * p.M * p.Nq;
     for (int w = blockIdx.x; w < n_pad_work; w += gridDim.x) {
         const int bm = w / p.Nq, head = w - bm * p.Nq;
         const int b = bm / p.M, mm = bm - b * p.M;
         const int st = pv.start[bm], ln = pv.len[bm];
+        if (ln != 0 && mm > 0 && mm < p.M - 1 && !(p.queue_view == 1 && fused[b] != 0)) continue;
         const int npad = p.H - ln;
         constexpr int CP8 = D / 8;
         __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
