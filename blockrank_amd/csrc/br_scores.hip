@@ -242,7 +242,10 @@ struct BrTileScoreParams {
     float out_scale;
 };
 
-__global__ __launch_bounds__(1024) void br_doc_final_tiles_kernel(BrTileScoreParams p) {
+// MAXT: threads per workgroup the instance is compiled for (1024: sixteen waves of at most 128 registers, for
+// the one-document-per-lane case; 512: eight waves of up to 256 registers, whose loads are all in flight together).
+template <int MAXT>
+__global__ __launch_bounds__(MAXT) void br_doc_final_tiles_kernel(BrTileScoreParams p) {
     extern __shared__ float dyn[];      // [nwaves][docs]
     const int docs = p.M - 2;
     const int b = blockIdx.x;
@@ -307,7 +310,98 @@ __global__ __launch_bounds__(1024) void br_doc_final_tiles_kernel(BrTileScorePar
             }
         }
     }
-    for (int j = wave; j < NR && !small; j += nwaves) {
+    // Up to 256 documents of at most 8 tiles: a lane takes documents lane, lane + 64, ...; each document's
+    // tiles are reduced to (max, sum) as they arrive, two (head, row) pairs of a wave at a time.
+    const bool medium = !small && docs <= 256 && p.H <= 8 * BR_BN;
+    if (medium) {
+        constexpr int PG = 4, DPL = 4;
+        const int kmax = (docs + 63) >> 6;       // document slots per lane actually in use
+        int t0m[DPL], ntm[DPL];
+#pragma unroll
+        for (int k = 0; k < DPL; ++k) {
+            const int d = lane + 64 * k;
+            t0m[k] = d < docs ? tbase[b * p.M + d + 1] : 0;
+            ntm[k] = d < docs ? (len[b * p.M + d + 1] + BR_BN - 1) / BR_BN : 0;
+        }
+        for (int j0 = wave; j0 < NR; j0 += PG * nwaves) {
+            float md[PG][DPL], sdm[PG][DPL];
+            bool pair_on[PG];
+            const float2* base[PG];
+            bool row_ok[PG];
+#pragma unroll
+            for (int i = 0; i < PG; ++i) {
+                const int j = j0 + i * nwaves;
+                pair_on[i] = j < NR;
+                const int jj = pair_on[i] ? j : 0;
+                const int n = jj / p.R, r = jj - n * p.R;
+                int r16 = p.rows[b * p.R + r];
+                r16 = r16 < 0 ? 0 : (r16 >= p.Rw ? p.Rw - 1 : r16);
+                const int pos = p.H - p.Rw + r16;
+                row_ok[i] = pair_on[i] && pos >= st_q && pos < st_q + len_q;
+                base[i] = reinterpret_cast<const float2*>(p.part) + (((long long)b * p.Nq + n) * p.Rw + r16) * tps;
+            }
+#pragma unroll
+            for (int k = 0; k < DPL; ++k) {
+#pragma unroll
+                for (int i = 0; i < PG; ++i) {
+                    md[i][k] = -INFINITY;
+                    sdm[i][k] = 0.f;
+                }
+                if (k >= kmax) continue;
+                float2 v[PG][8];
+#pragma unroll
+                for (int i = 0; i < PG; ++i)
+#pragma unroll
+                    for (int t8 = 0; t8 < 8; ++t8) v[i][t8] = base[i][t0m[k] + (t8 < ntm[k] ? t8 : 0)];   // always a valid address
+#pragma unroll
+                for (int i = 0; i < PG; ++i)
+#pragma unroll
+                    for (int t8 = 0; t8 < 8; ++t8)
+                        if (!(row_ok[i] && t8 < ntm[k])) v[i][t8] = make_float2(-INFINITY, 0.f);
+#pragma unroll
+                for (int i = 0; i < PG; ++i) {
+                    float m = -INFINITY;
+#pragma unroll
+                    for (int t8 = 0; t8 < 8; ++t8) m = fmaxf(m, v[i][t8].x);
+                    float sacc = 0.f;
+#pragma unroll
+                    for (int t8 = 0; t8 < 8; ++t8)
+                        if (v[i][t8].x != -INFINITY) sacc += v[i][t8].y * __builtin_amdgcn_exp2f(v[i][t8].x - m);
+                    md[i][k] = m;
+                    sdm[i][k] = sacc;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < PG; ++i) {
+                if (!pair_on[i]) continue;
+                const int j = j0 + i * nwaves;
+                float* pr_out = p.probs ? p.probs + ((long long)b * NR + j) * docs : nullptr;
+                float mx = -INFINITY;
+#pragma unroll
+                for (int k = 0; k < DPL; ++k) mx = fmaxf(mx, md[i][k]);
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+                float den = 0.f;
+#pragma unroll
+                for (int k = 0; k < DPL; ++k) {
+                    sdm[i][k] = md[i][k] == -INFINITY ? 0.f : sdm[i][k] * __builtin_amdgcn_exp2f(md[i][k] - mx);
+                    den += sdm[i][k];
+                }
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
+#pragma unroll
+                for (int k = 0; k < DPL; ++k) {
+                    const int d = lane + 64 * k;
+                    if (d < docs) {
+                        const float pr = den > 0.f ? sdm[i][k] / den : uniform;
+                        if (pr_out) pr_out[d] = pr;
+                        mine[d] += pr;
+                    }
+                }
+            }
+        }
+    }
+    for (int j = wave; j < NR && !small && !medium; j += nwaves) {
         const int n = j / p.R, r = j - n * p.R;
         int r16 = p.rows[b * p.R + r];
         r16 = r16 < 0 ? 0 : (r16 >= p.Rw ? p.Rw - 1 : r16);
@@ -477,10 +571,14 @@ int br_launch_doc_scores_tiles(const float* part, const int* plan, const int* ro
     p.part = part; p.plan = plan; p.rows = rows; p.scores = scores; p.probs = probs;
     p.B = B; p.Nq = Nq; p.M = M; p.H = H; p.R = R; p.Rw = Rw; p.out_scale = out_scale;
     const int docs = M - 2;
-    int nwaves = 16;
+    const bool small = docs <= 64 && H <= 8 * BR_BN;      // the kernel's own test for its one-document-per-lane path
+    int nwaves = small ? 16 : 8;
     while (nwaves > 1 && (size_t)nwaves * docs * sizeof(float) > 48 * 1024) nwaves >>= 1;
     if ((size_t)nwaves * docs * sizeof(float) > 60 * 1024) return 1;
-    hipLaunchKernelGGL(br_doc_final_tiles_kernel, dim3(B), dim3(nwaves * 64), (size_t)nwaves * docs * sizeof(float), stream, p);
+    if (small)
+        hipLaunchKernelGGL(br_doc_final_tiles_kernel<1024>, dim3(B), dim3(nwaves * 64), (size_t)nwaves * docs * sizeof(float), stream, p);
+    else
+        hipLaunchKernelGGL(br_doc_final_tiles_kernel<512>, dim3(B), dim3(nwaves * 64), (size_t)nwaves * docs * sizeof(float), stream, p);
     return 0;
 }
 
