@@ -58,6 +58,9 @@ def workloads():
         # one long causal block per sequence: many key tiles per work item (steady-state tile throughput)
         "causal4k": dict(desc="single block of 4096 tokens per sequence (plain causal), B=8, 32q/8kv heads, D=128, bf16",
                          layout=lambda: synthetic.make_layout([[4096]] * 8), Nq=32, Nkv=8, D=128, hidden=None, dtype=torch.bfloat16),
+        # the headline layout with eight query heads per kv head (Llama-3-70B-like grouping)
+        "cfg2g8": dict(desc="cfg2 layout with 32q/4kv heads (8 per group), D=128, bf16", layout=lambda: synthetic.uniform_layout(4, 64, 20, 160, 32),
+                       Nq=32, Nkv=4, D=128, hidden=None, dtype=torch.bfloat16),
         # BASELINE configs[0]: the reference's CPU-runnable case
         "cfg1": dict(desc="fp32, B=1, 8q/2kv heads, D=64, 32-token prefix + 8 docs x 64 + 16-token query", layout=lambda: synthetic.uniform_layout(1, 32, 8, 64, 16),
                      Nq=8, Nkv=2, D=64, hidden=None, dtype=torch.float32),

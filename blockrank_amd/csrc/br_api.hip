@@ -44,8 +44,10 @@ int fail(int code, const char* fmt, ...) {
 bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW) {
     if (Nq <= 0 || Nkv <= 0 || Nq % Nkv) return false;
     const int G = Nq / Nkv;
+    // experiment knob: BLOCKRANK_MAX_GW caps the heads one workgroup covers
+    static const int max_gw = getenv("BLOCKRANK_MAX_GW") ? atoi(getenv("BLOCKRANK_MAX_GW")) : 8;
     int Gw = 1;
-    for (int d = 1; d <= 8 && d <= G; ++d)
+    for (int d = 1; d <= 8 && d <= G && d <= max_gw; ++d)
         if (G % d == 0) Gw = d;
     int nw, tpb;
     switch (Gw) {
