@@ -134,6 +134,8 @@ def bench_model(args):
     R = min(16, layout.H)
     rows = torch.tensor([[R - 2, R - 1]] * B, dtype=torch.int32, device=dev)
     ranker = br.TruncatedRanker(model, layer_idx)
+    if not args.hf_rope:
+        br.patch_rotary(model)           # the one-pass rotary embedding kernel instead of the model file's eager expression
     steps = args.steps if args.steps is not None else 10
     warmup = args.warmup if args.warmup is not None else 2
     if args.padded:
@@ -181,7 +183,8 @@ def bench_model(args):
                                "layers 0..19 in full and the score part of layer 20, bf16",
                    "name": "cfg3", "batch": B, "blocks": layout.M, "block_len": layout.H, "valid_tokens": layout.valid_tokens,
                    "padded_tokens": B * S, "unmasked_pairs": pairs_n, "launch": "eager",
-                   "token_layout": "padded (B, M, H)" if args.padded else "packed (real tokens only)"},
+                   "token_layout": "padded (B, M, H)" if args.padded else "packed (real tokens only)",
+                   "rotary": "model's eager expression" if args.hf_rope else "one-pass HIP kernel"},
         "prefill_tok_per_s": layout.valid_tokens / (ms_per_step * 1e-3),
         "attention_ms_per_step": sum(kern_ms),
         "attention_share": sum(kern_ms) / ms_per_step,
@@ -206,6 +209,7 @@ def main():
     ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
     ap.add_argument("--qk-fp8", action="store_true",
                     help="compute Q K^T in fp8 e4m3 (bf16 workloads with head dim 128; includes the quantisation pass)")
+    ap.add_argument("--hf-rope", action="store_true", help="cfg3: keep the model file's own rotary embedding (eight elementwise passes per layer)")
     ap.add_argument("--padded", action="store_true",
                     help="cfg3: feed the reference's padded (B, M, H) batch instead of the packed one")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -26,8 +26,12 @@ from .attention import (
 from .losses import compute_auxiliary_attention_loss, rank_documents
 from .ranker import TruncatedRanker
 from .collate import block_icr_collate_packed, pack_padded_batch
+from .rope import apply_rotary_pos_emb, patch_rotary, unpatch_rotary
 
 __all__ = [
+    "apply_rotary_pos_emb",
+    "patch_rotary",
+    "unpatch_rotary",
     "BlockMask",
     "LastBlockScores",
     "blockrank_attention",

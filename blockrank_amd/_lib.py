@@ -51,6 +51,8 @@ SIGNATURES = {
                               c_void_p, c_void_p, c_float, c_float, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "br_last_block_logits": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_float, c_float, c_int, c_void_p, c_void_p]),
+    "br_rope_qk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                           c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
 
 _lib = None

@@ -21,6 +21,8 @@ int br_launch_prefill_fp8qk(const BrPrefillParams& p, int D, int NW, int n_cu, i
 void br_launch_quantize_fp8(const void* q, const void* k, const int* plan, void* q8, void* k8, unsigned* amax, float* scales,
                             const long long* sq, const long long* sk, long long q8_b, long long q8_h, long long k8_b, long long k8_h,
                             int B, int Nq, int Nkv, int M, int H, int D, hipStream_t stream);
+int br_launch_rope(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
+                   int D, const long long* sq, const long long* sk, const long long* sc, int dtype, int n_cu, hipStream_t stream);
 int br_launch_doc_scores_tiles(const float* part, const int* plan, const int* rows, float* scores, float* probs, int B, int Nq,
                                int M, int H, int R, int Rw, float out_scale, hipStream_t stream);
 int br_launch_last_logits(const void* q, const void* k, const int* plan, const int* rows, float* logits, const long long* sq,
@@ -394,6 +396,27 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
     br_launch_last_logits(q, k, plan, rows, logits, sq, sk, B, Nq, Nkv, M, H, D, R, br_tokens_per_tile(g), scale, neg,
                           dtype, static_cast<hipStream_t>(stream));
     return check_launch("logits launch");
+}
+
+int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
+               int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* cs_strides, int dtype, void* stream) {
+    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "dtype must be fp32 (0) or bf16 (1)");
+    if (B <= 0 || Nq <= 0 || Nkv <= 0 || S <= 0) return fail(BR_ERR_ARG, "B, Nq, Nkv and S must be positive");
+    if (D != 64 && D != 128) return fail(BR_ERR_ARG, "head dim %d not supported (64 or 128)", D);
+    if (!q || !k || !cos || !sin || !q_out || !k_out || !q_strides || !k_strides || !cs_strides) return fail(BR_ERR_ARG, "null pointer");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(cos) || !aligned16(sin) || !aligned16(q_out) || !aligned16(k_out))
+        return fail(BR_ERR_ARG, "q, k, cos, sin and the outputs must be 16-byte aligned");
+    int rc;
+    if ((rc = check_strides("q", q_strides, dtype)) || (rc = check_strides("k", k_strides, dtype))) return rc;
+    const int per16 = dtype == BR_DTYPE_F32 ? 4 : 8;
+    if (cs_strides[0] % per16 || cs_strides[1] % per16 || cs_strides[0] < 0 || cs_strides[1] < 0)
+        return fail(BR_ERR_ARG, "cos/sin strides must be non-negative multiples of 16 bytes");
+    const int n_cu = n_compute_units();
+    if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
+    const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]}, sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
+    const long long sc[2] = {cs_strides[0], cs_strides[1]};
+    br_launch_rope(q, k, cos, sin, q_out, k_out, B, Nq, Nkv, S, D, sq, sk, sc, dtype, n_cu, static_cast<hipStream_t>(stream));
+    return check_launch("rotary embedding launch");
 }
 
 }  // extern "C"

@@ -1,0 +1,68 @@
+"""Rotary position embedding of Q and K in one HIP pass.
+
+``apply_rotary_pos_emb`` has the signature and the result layout of the function of the same name in the
+Hugging Face model files (transformers models/mistral/modeling_mistral.py, and the Llama / Qwen2 copies),
+which every decoder layer of the models BlockRank ranks with calls on the projected Q and K right before
+the attention interface.  There it is eight elementwise passes per layer (measured at the Mistral-7B
+shape: 9 % of a ranking forward); here Q and K are read once and written once.  ``patch_rotary`` swaps
+it into the module a model's attention class was defined in; ``TruncatedRanker`` then uses it as well.
+"""
+from __future__ import annotations
+
+import sys
+
+import torch
+
+from . import _lib
+from .attention import _DTYPE_CODE, _dense_last_dim, _stream_ptr
+
+_I64x2 = _lib.ctypes.c_int64 * 2
+
+
+def apply_rotary_pos_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqueeze_dim: int = 1):
+    """q (B, Nq, S, D), k (B, Nkv, S, D) (any strides with a dense last dim, e.g. the head-transposed views of
+    the projections), cos / sin (B or 1, S, D).  Returns (q_embed, k_embed) with the same logical shapes, stored
+    as (B, S, heads, D) - what the attention hook takes without a copy.  bf16 or fp32, D 64 or 128, CUDA tensors."""
+    assert unsqueeze_dim == 1, "only the (batch, heads, tokens, dim) convention of the decoder layers is supported"
+    assert q.is_cuda and k.is_cuda and cos.is_cuda and sin.is_cuda, "the rotary embedding kernel needs device tensors"
+    assert q.dtype == k.dtype == cos.dtype == sin.dtype and q.dtype in _DTYPE_CODE, "q, k, cos and sin must share a dtype (bf16 or fp32)"
+    B, Nq, S, D = q.shape
+    Nkv = k.shape[1]
+    assert k.shape == (B, Nkv, S, D) and cos.shape[-2:] == (S, D) and sin.shape == cos.shape and cos.dim() == 3
+    assert cos.shape[0] in (1, B), "cos/sin must have the batch size of q or 1"
+    lib = _lib.load()
+    per16 = 16 // q.element_size()
+    q = _dense_last_dim(q, per16)
+    k = _dense_last_dim(k, per16)
+    if cos.stride(-1) != 1 or cos.stride(0) % per16 or cos.stride(1) % per16 or cos.stride() != sin.stride():
+        cos, sin = cos.contiguous(), sin.contiguous()
+    with torch.cuda.device(q.device):
+        q_out = torch.empty((B, S, Nq, D), dtype=q.dtype, device=q.device)
+        k_out = torch.empty((B, S, Nkv, D), dtype=q.dtype, device=q.device)
+        cs = _I64x2(0 if cos.shape[0] == 1 else cos.stride(0), cos.stride(1))
+        _lib.check(lib.br_rope_qk(q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(), q_out.data_ptr(), k_out.data_ptr(), B, Nq, Nkv,
+                                  S, D, _lib.strides3(q), _lib.strides3(k), cs, _DTYPE_CODE[q.dtype], _stream_ptr(q.device)))
+    return q_out.transpose(1, 2), k_out.transpose(1, 2)
+
+
+def patch_rotary(model) -> list[str]:
+    """Replace ``apply_rotary_pos_emb`` in the module(s) that define the attention classes of ``model`` (a
+    Hugging Face decoder).  Returns the names of the patched modules; ``unpatch_rotary`` restores them."""
+    done = []
+    for m in model.modules():
+        mod = sys.modules.get(type(m).__module__)
+        if mod is None or mod.__name__ in done or not hasattr(mod, "apply_rotary_pos_emb") or not type(m).__name__.endswith("Attention"):
+            continue
+        if getattr(mod.apply_rotary_pos_emb, "__module__", "") != __name__:
+            mod._blockrank_amd_saved_rotary = mod.apply_rotary_pos_emb
+            mod.apply_rotary_pos_emb = apply_rotary_pos_emb
+        done.append(mod.__name__)
+    return done
+
+
+def unpatch_rotary(model) -> None:
+    for m in model.modules():
+        mod = sys.modules.get(type(m).__module__)
+        if mod is not None and hasattr(mod, "_blockrank_amd_saved_rotary"):
+            mod.apply_rotary_pos_emb = mod._blockrank_amd_saved_rotary
+            del mod._blockrank_amd_saved_rotary

@@ -178,6 +178,20 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
                          int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
                          float scale, float neg, int dtype, float* logits, void* stream);
 
+/* Rotary position embedding of Q and K in one pass, the step in front of every attention call:
+ * out = x * cos + rotate_half(x) * sin, rotate_half(x) = (-x[D/2:], x[:D/2]).  Replaces apply_rotary_pos_emb of
+ * the Hugging Face model the reference ranks with (transformers models/mistral/modeling_mistral.py,
+ * rotate_half and apply_rotary_pos_emb; the same function in the Llama and Qwen2 model files), which the
+ * reference reaches through the model forward of scripts/eval_attn.py:139-151 and scripts/train.py.
+ *   q (B, Nq, S, D), k (B, Nkv, S, D) logical, element strides (batch, head, token) as for br_prefill_fwd;
+ *   cos, sin (B, S, D) with element strides (batch, token) - a batch stride of 0 broadcasts one table;
+ *   q_out (B, S, Nq, D), k_out (B, S, Nkv, D) contiguous: the layout whose head-transposed views the
+ *   attention entry points take.  dtype 0 fp32, 1 bf16 for all six tensors; D 64 or 128.
+ * fp32 arithmetic with one rounding of the result (the reference's eager bf16 expression rounds every
+ * intermediate product and the sum). */
+int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
+               int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* cs_strides, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

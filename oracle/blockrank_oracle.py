@@ -24,6 +24,12 @@ How each function is pinned (see tests/test_oracle_*.py):
   doc_scores_from_logits           closed forms: q = 0 gives len_i / sum(len); scores * tau sum to
                                    1; permutation equivariance; hand-computed 2-document case.
   topk_indices                     definition (stable descending order).
+  rotary_embedding                 restates a third-party function the reference calls through the model
+                                   forward (transformers >= 4.30 per the reference's requirements.txt:3;
+                                   the installed 5.x has the same definition): pinned by the plane-rotation
+                                   closed form (angle 0 = identity, pair norms preserved, angle then minus
+                                   angle = identity, the vector (1, 0) goes to (cos, sin)) and against
+                                   complex multiplication.
 No golden vectors exist in the reference (it ships no tests); none of the functions above needed
 an import of the reference to be pinned, so the reference was only read, never run.
 """
@@ -353,3 +359,20 @@ def quantize_fp8_e4m3(x: torch.Tensor, valid: torch.Tensor) -> torch.Tensor:
     q = (xf / safe).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).float()
     return torch.where(keep, q * scale, torch.zeros((), dtype=torch.float32))
 
+
+# --------------------------------------------------------------------------------------------
+# the step in front of attention: rotary position embedding
+# --------------------------------------------------------------------------------------------
+
+def rotary_embedding(x: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+    """x (B, N, S, D); cos, sin (B or 1, S, D).  out = x * cos + rotate_half(x) * sin with
+    rotate_half(x) = concat(-x[..., D/2:], x[..., :D/2]) - the published definition in transformers
+    models/mistral/modeling_mistral.py (rotate_half, apply_rotary_pos_emb; identical in the Llama and Qwen2
+    files), which the reference applies through the Hugging Face model forward (scripts/eval_attn.py:139-151).
+    float64."""
+    x = np.asarray(x, dtype=np.float64)
+    c = np.asarray(cos, dtype=np.float64)[:, None]
+    s_ = np.asarray(sin, dtype=np.float64)[:, None]
+    h = x.shape[-1] // 2
+    rot = np.concatenate([-x[..., h:], x[..., :h]], axis=-1)
+    return x * c + rot * s_

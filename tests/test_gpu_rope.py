@@ -1,0 +1,93 @@
+"""The one-pass rotary embedding kernel: against the float64 oracle on the same inputs (fp32: 1e-6; bf16:
+the rounding of the result, 2^-8 relative), closer to it than the eager bf16 expression it replaces, and
+swapped into a small Hugging Face model without changing what the model computes."""
+import numpy as np
+import pytest
+import torch
+
+import blockrank_amd as br
+from blockrank_amd import synthetic
+from oracle import blockrank_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _inputs(B, Nq, Nkv, S, D, dtype, seed, batch_table=True):
+    g = torch.Generator().manual_seed(seed)
+    # head-transposed views of (B, S, heads, D) projections, as the decoder layers hand them over
+    q = torch.randn(B, S, Nq, D, generator=g).to(DEV, dtype).transpose(1, 2)
+    k = torch.randn(B, S, Nkv, D, generator=g).to(DEV, dtype).transpose(1, 2)
+    ang = torch.rand(B if batch_table else 1, S, D // 2, generator=g) * 6.28
+    ang = torch.cat([ang, ang], dim=-1)
+    return q, k, ang.cos().to(DEV, dtype), ang.sin().to(DEV, dtype)
+
+
+def _eager(q, k, cos, sin):
+    def rot(x):
+        h = x.shape[-1] // 2
+        return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+    c, s = cos.unsqueeze(1), sin.unsqueeze(1)
+    return q * c + rot(q) * s, k * c + rot(k) * s
+
+
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.float32, 128), (torch.bfloat16, 64), (torch.bfloat16, 128)])
+@pytest.mark.parametrize("batch_table", [True, False])
+def test_kernel_matches_the_oracle(dtype, D, batch_table):
+    B, Nq, Nkv, S = 2, 6, 2, 37
+    q, k, cos, sin = _inputs(B, Nq, Nkv, S, D, dtype, seed=D, batch_table=batch_table)
+    qo, ko = br.apply_rotary_pos_emb(q, k, cos, sin)
+    assert qo.shape == q.shape and ko.shape == k.shape and qo.dtype == dtype
+    assert qo.transpose(1, 2).is_contiguous() and ko.transpose(1, 2).is_contiguous()       # stored (B, S, heads, D)
+    c64, s64 = cos.double().cpu().numpy(), sin.double().cpu().numpy()
+    eq, ek = _eager(q, k, cos, sin)
+    for got, x, eager in ((qo, q, eq), (ko, k, ek)):
+        want = orc.rotary_embedding(x.double().cpu().numpy(), c64, s64)
+        err = np.abs(got.double().cpu().numpy() - want)
+        if dtype == torch.float32:
+            assert err.max() <= 1e-6
+        else:
+            assert (err <= 2.0 ** -8 * np.maximum(np.abs(want), 1e-2)).all(), err.max()
+            # one rounding instead of three: on average nearer the exact value than the eager expression
+            assert err.mean() <= np.abs(eager.double().cpu().numpy() - want).mean()
+
+
+def test_argument_errors():
+    q, k, cos, sin = _inputs(1, 2, 1, 8, 64, torch.bfloat16, seed=1)
+    with pytest.raises(AssertionError):
+        br.apply_rotary_pos_emb(q, k, cos.float(), sin.float())
+    with pytest.raises(AssertionError):
+        br.apply_rotary_pos_emb(q, k, cos[:, :4], sin[:, :4])
+    q96 = torch.randn(1, 2, 8, 96, device=DEV, dtype=torch.bfloat16)
+    c96 = torch.ones(1, 8, 96, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        br.apply_rotary_pos_emb(q96, q96, c96, c96)
+
+
+@pytest.mark.parametrize("kind", ["mistral", "qwen2"])
+def test_patched_model_and_ranker_agree_with_unpatched(kind):
+    from tests.test_gpu_hf_model import build
+    br.register_blockrank_attention()
+    model = build(kind, torch.bfloat16)
+    model.set_attn_implementation("sdpa_blockrank")
+    lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
+    ids = torch.randint(0, 512, (lay.B, lay.S), generator=torch.Generator().manual_seed(1)).to(DEV)
+    pos, valid, labels = lay.position_ids.to(DEV), lay.valid.to(DEV), lay.labels.to(DEV)
+    ranker = br.TruncatedRanker(model, layer_idx=2)
+    with torch.no_grad():
+        ref_h = model(input_ids=ids, position_ids=pos, attention_mask=valid, output_hidden_states=True, use_cache=False).hidden_states[-1]
+        ref_s = ranker(ids, valid, pos, labels)
+    names = br.patch_rotary(model)
+    try:
+        assert names and all(kind in n for n in names)
+        with torch.no_grad():
+            got_h = model(input_ids=ids, position_ids=pos, attention_mask=valid, output_hidden_states=True, use_cache=False).hidden_states[-1]
+            got_s = ranker(ids, valid, pos, labels)
+    finally:
+        br.unpatch_rotary(model)
+    rows = lay.valid.reshape(lay.B, lay.S).to(DEV)
+    assert (got_h.float() - ref_h.float())[rows].abs().max().item() <= 6e-2
+    torch.testing.assert_close(got_s, ref_s, rtol=2e-2, atol=2e-2)
+    import sys
+    mod = sys.modules[type(model.model.layers[0].self_attn).__module__]
+    assert mod.apply_rotary_pos_emb.__module__ != "blockrank_amd.rope", "unpatch_rotary must restore the model's own function"
