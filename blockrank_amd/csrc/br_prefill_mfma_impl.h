@@ -265,6 +265,11 @@ struct Prefill {
     static constexpr int JO = UNIFORM_STEP ? 1 : JK;
     static constexpr int JOK = UNIFORM_STEP ? 1 : JKK;
     static constexpr int STEP_ROWS = NW * 64 / CPR;        // rows between consecutive V pieces of a wave
+    // V swizzle: LDS piece = global piece ^ ((row & 3) << VSW).  One transposing read touches eight key rows
+    // (rows r, r+1, r+2, r+3 and the same eight rows further), 64 bytes of each: with 256-byte rows the four
+    // rows must land in four different 64-byte bank groups (shift 2); with 128-byte rows two rows share a bank
+    // line and the shift that separates them is 1.
+    static constexpr int VSW = CPR == 16 ? 2 : 1;
     static constexpr int STEP_ROWSK = NW * 64 / CPRK;      // ... K pieces
     struct Lane {
         int koff[JOK], voff[JO];   // global byte offsets inside a tile of this lane's DMA pieces
@@ -285,17 +290,16 @@ struct Prefill {
         for (int j = 0; j < JO; ++j) {
             const int slot = (wave + NW * j) * 64 + lane;
             const int prow = slot / CPR, cp = slot - prow * CPR;
-            L.voff[j] = prow * (int)p.v32_t * 2 + ((cp ^ ((prow & 3) << 1)) << 4);
+            L.voff[j] = prow * (int)p.v32_t * 2 + ((cp ^ ((prow & 3) << VSW)) << 4);
         }
         const int ln = lane & 31, lh = lane >> 5;
         if (F8) L.krd = ln * SM::rowKB + (((ln & (CPRK < 8 ? CPRK - 1 : 7))) << 4) + lh * 8;   // 8 bytes: dims 16c + 8lh .. +7
         else L.krd = ln * SM::rowKB + ((lh ^ (ln & 7)) << 4);
         // transposing read: within a group of 16 lanes, lane s points at key (s >> 2), dims 4 * (s & 3)
         const int s = lane & 15, ln_hi = (lane >> 4) & 1;
-        const int cl = (2 * ln_hi + ((s & 3) >> 1)) ^ ((s >> 2) << 1);
 #pragma unroll
         for (int d = 0; d < D / 32; ++d)
-            L.vrd[d] = SM::kBytes + (8 * lh + (s >> 2)) * SM::rowB + (((4 * d) ^ cl) << 4) + (s & 1) * 8;
+            L.vrd[d] = SM::kBytes + (8 * lh + (s >> 2)) * SM::rowB + (((4 * d + 2 * ln_hi + ((s & 3) >> 1)) ^ ((s >> 2) << VSW)) << 4) + (s & 1) * 8;
         return L;
     }
 
