@@ -1,0 +1,50 @@
+"""The attention + score step captured in a HIP graph: every replay must give the eager result, also with
+eager launches of the same library (which use and re-arm the same plan's ticket counters) in between.
+The library allocates nothing and records no memset: the plan's counters are re-armed by the last
+workgroup of each launch."""
+import pytest
+import torch
+
+import blockrank_amd as br
+from blockrank_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("resident", ["0", "1"])
+def test_graph_replays_equal_eager(resident, monkeypatch):
+    monkeypatch.setenv("BLOCKRANK_AMD_RESIDENT", resident)
+    lay = synthetic.make_layout([[40, 100, 160, 33, 192, 20], [64, 7, 150, 90, 0, 31]])
+    Nq, Nkv, D = 8, 2, 128
+    scale = D ** -0.5
+    q, k, v = synthetic.random_qkv(lay, Nq, Nkv, D, torch.bfloat16, DEV, seed=5)
+    mask = br.BlockMask(lay.valid.to(DEV), torch.bfloat16)
+    R = 16
+    rows = torch.tensor([[R - 2, R - 1]] * lay.B, dtype=torch.int32, device=DEV)
+
+    def step():
+        out, part = br.blockrank_attention(q, k, v, mask, scale, score_rows=R)
+        return out, br.doc_scores_from_partials(part, mask, rows, R, Nq, Nkv)
+
+    want_out, want_scores = step()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()                                   # warm-up on the capture stream
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=s):
+            g_out, g_scores = step()
+    torch.cuda.synchronize()
+    for i in range(4):
+        g_out.fill_(float("nan"))
+        g_scores.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_out, want_out), f"replay {i}: attention output differs from the eager result"
+        assert torch.equal(g_scores, want_scores), f"replay {i}: scores differ from the eager result"
+        e_out, e_scores = step()                 # eager work of the same kind between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(e_out, want_out) and torch.equal(e_scores, want_scores)
