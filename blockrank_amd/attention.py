@@ -220,6 +220,64 @@ def _dense_last_dim(t: torch.Tensor, per16: int) -> torch.Tensor:
     return t
 
 
+class _AttentionWithGrad(torch.autograd.Function):
+    """bf16 attention whose backward is the HIP kernel: the role of the reference's autograd-differentiated
+    hooks (blockrank_std_attention.py:96-262, :472-650, as trainer.py:79-101 uses them).  The forward saves
+    the log-sum-exp of every row; the backward rebuilds the probabilities from it."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, bm, scaling):
+        lib = _lib.load()
+        Bt, Nq, S, D = query.shape
+        Nkv = key.shape[1]
+        M, H, B, packed = bm.M, bm.H, bm.B, bm.packed
+        q, k, v = (_dense_last_dim(t.detach(), 8) for t in (query, key, value))
+        dev = query.device
+        with torch.cuda.device(dev):
+            plan = bm.plan(Nq, Nkv)
+            out = torch.empty((Bt, S, Nq, D), dtype=query.dtype, device=dev)
+            lse = torch.empty((Bt, Nq, S), dtype=torch.float32, device=dev)
+            ws_bytes = lib.br_prefill_workspace_bytes(B, Nq, Nkv, D)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+            _lib.check(lib.br_prefill_fwd_lse(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
+                _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed),
+                _lib._I64x3(0 if packed else S * Nq * D, D, Nq * D), scaling, ws.data_ptr(), ws_bytes, lse.data_ptr(),
+                _lib._I64x3(0 if packed else Nq * S, S, 1), _stream_ptr(dev)))
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.bm, ctx.scaling = bm, scaling
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        bm = ctx.bm
+        lib = _lib.load()
+        Bt, Nq, S, D = q.shape
+        Nkv = k.shape[1]
+        M, H, B, packed = bm.M, bm.H, bm.B, bm.packed
+        g = _dense_last_dim(dout.transpose(1, 2), 8)                     # logical (B, Nq, S, D)
+        dev = q.device
+        with torch.cuda.device(dev):
+            plan = bm.plan(Nq, Nkv)
+            dq = torch.empty((Bt, S, Nq, D), dtype=q.dtype, device=dev)
+            dk = torch.empty((Bt, S, Nkv, D), dtype=q.dtype, device=dev)
+            dv = torch.empty((Bt, S, Nkv, D), dtype=q.dtype, device=dev)
+            slots = Bt * S
+            ws_bytes = lib.br_prefill_bwd_workspace_bytes(Nq, Nkv, D, slots)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            bs = 0 if packed else 1
+            _lib.check(lib.br_prefill_bwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), g.data_ptr(), lse.data_ptr(), plan.data_ptr(),
+                B, Nq, Nkv, M, H, D,
+                _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed),
+                _lib._I64x3(bs * S * Nq * D, D, Nq * D), _lib.strides3(g, packed), _lib._I64x3(bs * Nq * S, S, 1),
+                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                _lib._I64x3(bs * S * Nq * D, D, Nq * D), _lib._I64x3(bs * S * Nkv * D, D, Nkv * D),
+                _lib._I64x3(bs * S * Nkv * D, D, Nkv * D), ctx.scaling, slots, ws.data_ptr(), ws_bytes, _stream_ptr(dev)))
+        return dq.transpose(1, 2), dk.transpose(1, 2), dv.transpose(1, 2), None, None
+
+
 def blockrank_attention(
     query: torch.Tensor,
     key: torch.Tensor,
@@ -264,8 +322,10 @@ def blockrank_attention(
         raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
     assert key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value must share a dtype"
     if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
-        # same contract as the reference's kernelised path (blockrank_triton_kernel_attention.py:759-761)
-        raise NotImplementedError("Backward pass not implemented yet")
+        if query.dtype != torch.bfloat16 or qk_fp8 or score_rows > 0:
+            # same contract as the reference's kernelised path (blockrank_triton_kernel_attention.py:759-761)
+            raise NotImplementedError("Backward pass not implemented yet (bfloat16 attention without fused score partials has one)")
+        return _AttentionWithGrad.apply(query, key, value, bm, float(scaling))
     lib = _lib.load()
     per16 = 16 // query.element_size()
     q = _dense_last_dim(query, per16)

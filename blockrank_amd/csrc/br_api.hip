@@ -29,6 +29,9 @@ int br_launch_last_logits(const void* q, const void* k, const int* plan, const i
                           const long long* sk, int B, int Nq, int Nkv, int M, int H, int D, int R, int T, float scale,
                           float neg, int dtype, hipStream_t stream);
 
+int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, void* dq, void* dk, void* dv, const long long* sdq, const long long* sdk,
+                  const long long* sdv, long long n_slots, long long slots_per_b, hipStream_t stream);
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -203,9 +206,10 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
                         int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                         const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
                         void* stream, void* ev_start, void* ev_stop, int score_rows, float* score_part, size_t score_part_bytes,
-                        int64_t fp8_tokens = 0) {
+                        int64_t fp8_tokens = 0, float* lse = nullptr, const int64_t* lse_strides = nullptr) {
     int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
     if (rc) return rc;
+    if (lse && (dtype != BR_DTYPE_BF16 || fp8_tokens > 0 || !lse_strides)) return fail(BR_ERR_ARG, "the log-sum-exp output comes from the bf16 kernel only");
     if (score_part) {
         if (dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "score partials come from the bf16 kernel only; use br_doc_scores");
         if (M < 3) return fail(BR_ERR_ARG, "score partials need at least one document block (M=%d)", M);
@@ -237,7 +241,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     // BLOCKRANK_AMD_RESIDENT=1, and only when the caller's workspace has that room: on the measured
     // workloads it does not beat the streaming kernel yet.
     const char* res_env = getenv("BLOCKRANK_AMD_RESIDENT");
-    const bool fused = dtype == BR_DTYPE_BF16 && fp8_tokens == 0 && (D == 64 || D == 128) && res_env && atoi(res_env) != 0 &&
+    const bool fused = dtype == BR_DTYPE_BF16 && fp8_tokens == 0 && !lse && (D == 64 || D == 128) && res_env && atoi(res_env) != 0 &&
                        workspace_bytes >= br_prefill_workspace_bytes_fused(B, M, Nq, Nkv, D);
     p.queue_view = fused ? 1 : 0;
     p.slots = fused ? br_slots_view1(M) : BR_SLOTS_PER_SEQ;
@@ -261,6 +265,9 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     p.score_part = score_part;
     p.score_R = score_part ? score_rows : 0;
     p.qk_scales = nullptr;
+    p.lse = lse;
+    p.lse_b = lse ? lse_strides[0] : 0;
+    p.lse_h = lse ? lse_strides[1] : 0;
     int combine_grid = br_plan_max_comb(B) * g.NHG;
     if (combine_grid < B * M) combine_grid = B * M;
     if (combine_grid > 4 * n_cu) combine_grid = 4 * n_cu;
@@ -332,6 +339,75 @@ int br_prefill_fwd_fp8qk(const void* q, const void* k, const void* v, void* out,
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale,
                         BR_DTYPE_BF16, workspace, workspace_bytes, stream, ev_start, ev_stop, score_rows, score_part,
                         score_part_bytes, tokens);
+}
+
+int br_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
+                       int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                       const int64_t* out_strides, float scale, void* workspace, size_t workspace_bytes, float* lse,
+                       const int64_t* lse_strides, void* stream) {
+    if (!lse || !lse_strides) return fail(BR_ERR_ARG, "lse and its strides must be provided");
+    if (lse_strides[0] < 0 || lse_strides[1] <= 0) return fail(BR_ERR_ARG, "bad lse strides");
+    return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, BR_DTYPE_BF16,
+                        workspace, workspace_bytes, stream, nullptr, nullptr, 0, nullptr, 0, 0, lse, lse_strides);
+}
+
+size_t br_prefill_bwd_workspace_bytes(int Nq, int Nkv, int D, int64_t token_slots) {
+    if (Nq <= 0 || Nkv <= 0 || D <= 0 || token_slots <= 0) return 0;
+    return (size_t)token_slots * (size_t)(Nq + 2 * Nkv) * D * sizeof(float);
+}
+
+int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+                   const int32_t* plan, int B, int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides,
+                   const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides, const int64_t* dout_strides,
+                   const int64_t* lse_strides, void* dq, void* dk, void* dv, const int64_t* dq_strides, const int64_t* dk_strides,
+                   const int64_t* dv_strides, float scale, int64_t token_slots, void* workspace, size_t workspace_bytes,
+                   void* stream) {
+    int rc = check_common(B, Nq, Nkv, M, H, D, BR_DTYPE_BF16);
+    if (rc) return rc;
+    if (!q || !k || !v || !out || !dout || !lse || !plan || !dq || !dk || !dv || !lse_strides) return fail(BR_ERR_ARG, "null pointer");
+    for (const void* ptr : {q, k, v, out, dout, (const void*)plan, (const void*)dq, (const void*)dk, (const void*)dv, (const void*)workspace})
+        if (!aligned16(ptr)) return fail(BR_ERR_ARG, "tensors, plan and workspace must be 16-byte aligned");
+    const int64_t* all[8] = {q_strides, k_strides, v_strides, out_strides, dout_strides, dq_strides, dk_strides, dv_strides};
+    const char* names[8] = {"q", "k", "v", "out", "dout", "dq", "dk", "dv"};
+    for (int i = 0; i < 8; ++i) {
+        if ((rc = check_strides(names[i], all[i], BR_DTYPE_BF16))) return rc;
+        for (int j = 0; j < 3; ++j)
+            if (all[i][j] >= (int64_t(1) << 31)) return fail(BR_ERR_ARG, "strides must be below 2^31 elements (got %lld)", (long long)all[i][j]);
+    }
+    if (lse_strides[0] < 0 || lse_strides[1] <= 0) return fail(BR_ERR_ARG, "bad lse strides");
+    const bool packed = q_strides[0] == 0;
+    if (!packed && token_slots != (int64_t)B * M * H) return fail(BR_ERR_ARG, "token_slots=%lld, expected B*M*H=%lld", (long long)token_slots, (long long)B * M * H);
+    if (token_slots <= 0) return fail(BR_ERR_ARG, "token_slots must be positive");
+    const size_t need = br_prefill_bwd_workspace_bytes(Nq, Nkv, D, token_slots);
+    if (!workspace || workspace_bytes < need) return fail(BR_ERR_SPACE, "workspace holds %zu bytes, %zu needed", workspace_bytes, need);
+    const int n_cu = n_compute_units();
+    if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
+    BrGeom g;
+    int nw;
+    make_geom(Nq, Nkv, &g, &nw);
+    BrBwdParams p;
+    p.q = q; p.k = k; p.v = v; p.out = out; p.dout = dout; p.plan = plan; p.lse = lse;
+    p.lse_b = lse_strides[0]; p.lse_h = lse_strides[1];
+    p.dq32 = static_cast<float*>(workspace);
+    p.dk32 = p.dq32 + (size_t)token_slots * Nq * D;
+    p.dv32 = p.dk32 + (size_t)token_slots * Nkv * D;
+    p.acc_b = packed ? 0 : (long long)M * H;
+    p.q32_b = (unsigned)q_strides[0]; p.q32_h = (unsigned)q_strides[1]; p.q32_t = (unsigned)q_strides[2];
+    p.k32_b = (unsigned)k_strides[0]; p.k32_h = (unsigned)k_strides[1]; p.k32_t = (unsigned)k_strides[2];
+    p.v32_b = (unsigned)v_strides[0]; p.v32_h = (unsigned)v_strides[1]; p.v32_t = (unsigned)v_strides[2];
+    p.o32_b = (unsigned)out_strides[0]; p.o32_h = (unsigned)out_strides[1]; p.o32_t = (unsigned)out_strides[2];
+    p.g32_b = (unsigned)dout_strides[0]; p.g32_h = (unsigned)dout_strides[1]; p.g32_t = (unsigned)dout_strides[2];
+    p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H;
+    p.geom = g;
+    p.scale = scale;
+    p.scale_log2 = scale * 1.4426950408889634f;
+    p.max_items = br_plan_max_items_view0(B, M, H, br_tokens_per_tile(g));
+    const long long sdq[3] = {dq_strides[0], dq_strides[1], dq_strides[2]}, sdk[3] = {dk_strides[0], dk_strides[1], dk_strides[2]},
+                    sdv[3] = {dv_strides[0], dv_strides[1], dv_strides[2]};
+    const int lrc = br_launch_bwd(p, D, nw, n_cu, dq, dk, dv, sdq, sdk, sdv, token_slots, packed ? 0 : (long long)M * H,
+                                  static_cast<hipStream_t>(stream));
+    if (lrc) return fail(BR_ERR_ARG, "no backward kernel for head dim %d with %d query heads per kv head (code %d)", D, g.G, lrc);
+    return check_launch("backward launch");
 }
 
 int br_doc_scores_from_partials(const float* score_part, const int32_t* plan, const int32_t* rows, int R, int score_rows, int B,

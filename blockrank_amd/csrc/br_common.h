@@ -99,6 +99,12 @@ __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
     int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
     return B * (2 * ((M > 1 ? (M - 1) * qt : 0) + last) + M);
 }
+// Upper bound on the items of view 0 alone (they are the first items of the array).
+__host__ __device__ inline int br_plan_max_items_view0(int B, int M, int H, int T) {
+    int qt = (H + T - 1) / T;
+    int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
+    return B * ((M > 1 ? (M - 1) * qt : 0) + last);
+}
 __host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }   // per view
 // Partial slots per sequence in view 1: a fused sequence uses (query tile, block) -> tile * M + block, two tiles at most.
 __host__ __device__ inline int br_slots_view1(int M) { return 2 * M > BR_SLOTS_PER_SEQ ? 2 * M : BR_SLOTS_PER_SEQ; }
@@ -281,4 +287,30 @@ struct BrPrefillParams {
     // fused sequences are left to the resident kernel
     int queue_view;
     int slots;         // partial slots per sequence (BR_SLOTS_PER_SEQ in view 0, br_slots_view1(M) in view 1)
+    // Optional: the log-sum-exp of every real query row, in base-2 units (log2 of the sum over the visible keys
+    // of 2^(scale * log2(e) * q.k)), at lse[b * lse_b + head * lse_h + token]; the backward pass starts from it.
+    // Null: not wanted.  Written by the streaming bf16 kernel and the finish kernel only.
+    float* lse;
+    long long lse_b, lse_h;
+};
+
+// Arguments of the backward kernel (bf16).
+struct BrBwdParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* out;
+    const void* dout;
+    const int* plan;
+    const float* lse;          // base-2 log-sum-exp of every real row, as the forward wrote it
+    long long lse_b, lse_h;
+    float* dq32;               // [slot][Nq][D] fp32, slot = b * acc_b + token
+    float* dk32;               // [slot][Nkv][D]
+    float* dv32;
+    long long acc_b;           // token slots per batch entry (0 for a packed layout: tokens are batch-global)
+    unsigned q32_b, q32_h, q32_t, k32_b, k32_h, k32_t, v32_b, v32_h, v32_t, o32_b, o32_h, o32_t, g32_b, g32_h, g32_t;
+    int B, Nq, Nkv, M, H;
+    BrGeom geom;
+    float scale, scale_log2;
+    int max_items;
 };

@@ -670,6 +670,8 @@ struct Prefill {
             // through LDS so that every output row is written as full 16-byte pieces
             __bf16* Es = reinterpret_cast<__bf16*>(smem + wave * SM::eBytesPerWave);
             const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;
+            if (p.lse != nullptr && lane_e < 32 && row0 + lane_e < len_m)
+                p.lse[(long long)b * p.lse_b + (long long)head * p.lse_h + qtok0 + row0 + lane_e] = m_run + __builtin_amdgcn_logf(l_tot);
             if (rb_active) {
 #pragma unroll
                 for (int d = 0; d < D / 32; ++d)
@@ -1098,6 +1100,8 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
             }
         }
         const float inv = l > 0.f ? 1.f / l : 0.f;
+        if (p.lse != nullptr && cc == 0)
+            p.lse[(long long)c.b * p.lse_b + (long long)head * p.lse_h + qtok0 + row] = mmax + __builtin_amdgcn_logf(l);
         __bf16* dst = reinterpret_cast<__bf16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
                       (long long)(qtok0 + row) * p.so_t;
         bf16x4 h4 = __builtin_convertvector(acc * inv, bf16x4);

@@ -192,6 +192,40 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
 int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
                int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* cs_strides, int dtype, void* stream);
 
+/* ---- training: forward that also saves the log-sum-exp, and the backward ----
+ * The reference trains through its torch hooks ("default_blockrank" and relatives,
+ * blockrank_std_attention.py:96-262 and :472-650, called by the aux-loss trainer, trainer.py:79-101), which
+ * torch autograd differentiates; its Triton hook raises NotImplementedError on backward
+ * (blockrank_triton_kernel_attention.py:759-761).  These two entry points are the hand-written counterpart.
+ *
+ * br_prefill_fwd_lse: br_prefill_fwd for bf16 tensors that also writes, for every real query token,
+ *   lse[b * lse_strides[0] + head * lse_strides[1] + token] = log2( sum over visible keys of 2^(scale*log2(e)*q.k) )
+ * (the natural log-sum-exp is lse * ln 2).  token is the index on the token axis of q (m*H + position for the
+ * padded layout, the running token index for a packed one, whose lse_strides[0] is 0).  Padded slots are not written.
+ */
+int br_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
+                       int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                       const int64_t* out_strides, float scale, void* workspace, size_t workspace_bytes, float* lse,
+                       const int64_t* lse_strides, void* stream);
+
+/* Bytes of scratch br_prefill_bwd needs (fp32 accumulators of dq, dk, dv).  token_slots = B*M*H for the padded
+ * layout, the packed token count otherwise. */
+size_t br_prefill_bwd_workspace_bytes(int Nq, int Nkv, int D, int64_t token_slots);
+
+/* Gradients of the attention output with respect to q, k and v (bf16, D 64 or 128):
+ *   P = softmax(scale * q.k over visible keys),  dV = P^T dO,  dS = P * (dO V^T - rowsum(dO * O)),
+ *   dQ = scale * dS K,  dK = scale * dS^T Q,  dK and dV summed over the query heads of a kv head.
+ * q, k, v, out, lse and plan exactly as given to / written by br_prefill_fwd_lse; dout has out's logical shape
+ * (B, Nq, S, D) with its own strides; dq (B, Nq, S, D), dk, dv (B, Nkv, S, D) with their strides.  Rows of padded
+ * slots receive zeros; dout on padded slots is ignored.  Sums are accumulated in fp32 with atomic adds, so the
+ * last bits depend on the order in which workgroups finish. */
+int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+                   const int32_t* plan, int B, int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides,
+                   const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides, const int64_t* dout_strides,
+                   const int64_t* lse_strides, void* dq, void* dk, void* dv, const int64_t* dq_strides, const int64_t* dk_strides,
+                   const int64_t* dv_strides, float scale, int64_t token_slots, void* workspace, size_t workspace_bytes,
+                   void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -19,6 +19,10 @@ How each function is pinned (see tests/test_oracle_*.py):
                                    SDPA on the concatenated valid tokens (no mask tensor at all),
                                    and by invariants (V = 1, document permutation, GQA expansion,
                                    garbage in padding).
+  dense_attention_backward         closed-form gradients; checked against central finite differences of
+                                   dense_attention in float64 and against torch autograd through
+                                   sdpa_blockrank_forward (library SDPA calls only); the log-sum-exp against
+                                   the rows of dense logits.
   last_block_logits                closed form scale*q.k + {0 | NEG}; checked against the rows of
                                    dense logits.
   doc_scores_from_logits           closed forms: q = 0 gives len_i / sum(len); scores * tau sum to
@@ -182,6 +186,52 @@ def dense_attention(q, k, v, valid, scale: float) -> Tuple[np.ndarray, np.ndarra
             p = e / e.sum(axis=1, keepdims=True)
             out[b, rows, n] = p @ vv
     return out, logits
+
+
+def dense_attention_backward(q, k, v, dout, valid, scale: float) -> Tuple[np.ndarray, np.ndarray, np.ndarray, np.ndarray]:
+    """Gradients of dense_attention in float64, in closed form, plus the log-sum-exp of every real row.
+
+    The reference has no hand-written backward: its trainable path (the "default"/"eager"/"sdpa" hooks,
+    blockrank_std_attention.py:96-262, :472-650, used by trainer.py:79-101) is differentiated by torch
+    autograd, and its Triton path refuses (blockrank_triton_kernel_attention.py:759-761).  This is the
+    derivative of softmax(scale*QK^T over allowed keys) V that autograd would produce:
+        P = softmax(S),  dV = P^T dO,  dP = dO V^T,  dS = P * (dP - rowsum(dP * P)),
+        dQ = scale * dS K,  dK = scale * dS^T Q,
+    with dK and dV summed over the query heads that share a kv head (the transpose of repeat_kv).
+    Rows of padded query tokens take part in nothing (their dout is ignored, their dq is zero).
+
+    q (B,Nq,S,D), k/v (B,Nkv,S,D), dout (B,S,Nq,D); returns dq (B,Nq,S,D), dk, dv (B,Nkv,S,D) and
+    lse (B,Nq,S) = log sum_j exp(scale*q.k_j) over allowed keys (NaN on padded rows).
+    """
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    dout = np.asarray(dout, dtype=np.float64)
+    B, Nq, S, D = q.shape
+    Nkv = k.shape[1]
+    G = Nq // Nkv
+    ok = allowed(valid)
+    dq = np.zeros_like(q)
+    dk = np.zeros_like(k)
+    dv = np.zeros_like(v)
+    lse = np.full((B, Nq, S), np.nan)
+    for b in range(B):
+        rows = ok[b].any(axis=1)
+        for n in range(Nq):
+            kk, vv = k[b, n // G], v[b, n // G]
+            s = np.where(ok[b][rows], scale * (q[b, n, rows] @ kk.T), -np.inf)
+            mx = s.max(axis=1, keepdims=True)
+            e = np.exp(s - mx)
+            den = e.sum(axis=1, keepdims=True)
+            p = e / den
+            lse[b, n, rows] = (mx + np.log(den))[:, 0]
+            do = dout[b, rows, n]
+            dv[b, n // G] += p.T @ do
+            dp = do @ vv.T
+            ds = p * (dp - (dp * p).sum(axis=1, keepdims=True))
+            dq[b, n, rows] = scale * (ds @ kk)
+            dk[b, n // G] += scale * (ds.T @ q[b, n, rows])
+    return dq, dk, dv, lse
 
 
 def sdpa_blockrank_forward(
