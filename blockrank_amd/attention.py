@@ -264,7 +264,7 @@ class _AttentionWithGrad(torch.autograd.Function):
             dk = torch.empty((Bt, S, Nkv, D), dtype=q.dtype, device=dev)
             dv = torch.empty((Bt, S, Nkv, D), dtype=q.dtype, device=dev)
             slots = Bt * S
-            ws_bytes = lib.br_prefill_bwd_workspace_bytes(Nq, Nkv, D, slots)
+            ws_bytes = lib.br_prefill_bwd_workspace_bytes(B, Nq, Nkv, H, D, slots)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             bs = 0 if packed else 1
             _lib.check(lib.br_prefill_bwd(
@@ -431,10 +431,19 @@ class LastBlockScores:
         H = self.block_mask.H
         return (torch.arange(H - self.R, H, dtype=torch.int32, device=self.device)[None]).expand(self.shape[0], self.R).contiguous()
 
+    def needs_grad(self) -> bool:
+        return torch.is_grad_enabled() and (self.query.requires_grad or self.key.requires_grad)
+
     def dense(self, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        """(B, Nq, R, S) logits + additive mask, fp32 unless ``dtype`` is given."""
-        out = last_block_logits(self.query, self.key, self.block_mask, self._rows_default(),
-                                self.scaling if self.scaled else 1.0, neg=0.7 * torch.finfo(self.dtype).min)
+        """(B, Nq, R, S) logits + additive mask, fp32 unless ``dtype`` is given.  Differentiable with respect
+        to the layer's query and key when they require gradients (the auxiliary attention loss of
+        trainer.py:79-101 trains through this tensor)."""
+        scale = self.scaling if self.scaled else 1.0
+        neg = 0.7 * torch.finfo(self.dtype).min
+        if self.needs_grad():
+            out = _LastLogitsWithGrad.apply(self.query, self.key, self.block_mask, self._rows_default(), scale, neg)
+        else:
+            out = last_block_logits(self.query, self.key, self.block_mask, self._rows_default(), scale, neg=neg)
         return out if dtype is None else out.to(dtype)
 
     def doc_scores(self, rows: torch.Tensor, temperature: float = 0.05, head_reduce: str = "mean", row_reduce: str = "mean",
@@ -541,6 +550,36 @@ def last_block_logits(query, key, block_mask, rows, scaling: float, neg: Optiona
     return out
 
 
+class _LastLogitsWithGrad(torch.autograd.Function):
+    """last_block_logits with a backward: s[b,n,r,k] = scaling * q[b,n,row_r] . k[b,n//G,k] + constant, so
+    dq[row_r] = scaling * sum_k ds k and dk[k] = scaling * sum_{n in group, r} ds q[row_r] - two small products
+    over the R score rows, done with torch matmuls (padded layout only)."""
+
+    @staticmethod
+    def forward(ctx, query, key, bm, rows, scaling, neg):
+        if bm.packed:
+            raise NotImplementedError("gradients of the score logits need the padded (B, M, H) layout")
+        ctx.save_for_backward(query, key, rows)
+        ctx.bm, ctx.scaling = bm, float(scaling)
+        return last_block_logits(query.detach(), key.detach(), bm, rows, scaling, neg=neg)
+
+    @staticmethod
+    def backward(ctx, ds):
+        query, key, rows = ctx.saved_tensors
+        bm = ctx.bm
+        B, Nq, S, D = query.shape
+        Nkv = key.shape[1]
+        G, R = Nq // Nkv, rows.shape[1]
+        tok = ((bm.M - 1) * bm.H + rows.long())[:, None, :, None].expand(B, Nq, R, D)          # token index of each score row
+        ds5 = ds.float().reshape(B, Nkv, G, R, S)
+        q_rows = query.detach().gather(2, tok).float().reshape(B, Nkv, G, R, D)
+        dq_rows = ctx.scaling * torch.einsum("bkgrs,bksd->bkgrd", ds5, key.detach().float())
+        dk = ctx.scaling * torch.einsum("bkgrs,bkgrd->bksd", ds5, q_rows)
+        dq = torch.zeros((B, Nq, S, D), dtype=torch.float32, device=query.device)
+        dq.scatter_add_(2, tok, dq_rows.reshape(B, Nq, R, D))
+        return dq.to(query.dtype), dk.to(key.dtype), None, None, None, None
+
+
 def blockrank_attention_forward(
     module,
     query: torch.Tensor,
@@ -586,7 +625,11 @@ def blockrank_attention_forward(
     num_last = kwargs.get("num_last_queries", 16)
     R = num_last if bm.H >= num_last else bm.H
     scaled = not kwargs.get("unscaled_scores", False)
-    fuse = want and scaled and fused_scores_supported(query, bm) and not _env_flag("BLOCKRANK_AMD_SEPARATE_SCORES")
+    # training (gradients wanted): the attention runs through its autograd function and the scores come back
+    # as the dense, differentiable logits tensor the reference returns
+    needs_grad = torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad)
+    fuse = (want and scaled and not needs_grad and fused_scores_supported(query, bm)
+            and not _env_flag("BLOCKRANK_AMD_SEPARATE_SCORES"))
 
     qk_fp8 = bool(kwargs.get("qk_fp8", False)) or _env_flag("BLOCKRANK_AMD_QK_FP8")
     out = blockrank_attention(query, key, value, bm, scaling, kernel_events=kwargs.get("kernel_events", None),
@@ -597,7 +640,7 @@ def blockrank_attention_forward(
     if not want:
         return out, None
     handle = LastBlockScores(query, key, bm, scaling, R, scaled=scaled, partials=partials)
-    if kwargs.get("materialize_scores", False) or _env_flag("BLOCKRANK_AMD_DENSE_SCORES"):
+    if needs_grad or kwargs.get("materialize_scores", False) or _env_flag("BLOCKRANK_AMD_DENSE_SCORES"):
         return out, handle.dense()
     return out, handle
 

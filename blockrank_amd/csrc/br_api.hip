@@ -29,8 +29,7 @@ int br_launch_last_logits(const void* q, const void* k, const int* plan, const i
                           const long long* sk, int B, int Nq, int Nkv, int M, int H, int D, int R, int T, float scale,
                           float neg, int dtype, hipStream_t stream);
 
-int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, void* dq, void* dk, void* dv, const long long* sdq, const long long* sdk,
-                  const long long* sdv, long long n_slots, long long slots_per_b, hipStream_t stream);
+int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, hipStream_t stream);
 
 namespace {
 
@@ -351,9 +350,10 @@ int br_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, c
                         workspace, workspace_bytes, stream, nullptr, nullptr, 0, nullptr, 0, 0, lse, lse_strides);
 }
 
-size_t br_prefill_bwd_workspace_bytes(int Nq, int Nkv, int D, int64_t token_slots) {
-    if (Nq <= 0 || Nkv <= 0 || D <= 0 || token_slots <= 0) return 0;
-    return (size_t)token_slots * (size_t)(Nq + 2 * Nkv) * D * sizeof(float);
+size_t br_prefill_bwd_workspace_bytes(int B, int Nq, int Nkv, int H, int D, int64_t token_slots) {
+    if (B <= 0 || Nq <= 0 || Nkv <= 0 || H <= 0 || D <= 0 || token_slots <= 0) return 0;
+    // fp32 dQ sums of the query block's rows and dK, dV sums of the prefix keys, then delta for every token slot and query head
+    return up256((size_t)B * (Nq + 2 * Nkv) * H * D * sizeof(float)) + (size_t)token_slots * Nq * sizeof(float);
 }
 
 int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
@@ -378,20 +378,30 @@ int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out,
     const bool packed = q_strides[0] == 0;
     if (!packed && token_slots != (int64_t)B * M * H) return fail(BR_ERR_ARG, "token_slots=%lld, expected B*M*H=%lld", (long long)token_slots, (long long)B * M * H);
     if (token_slots <= 0) return fail(BR_ERR_ARG, "token_slots must be positive");
-    const size_t need = br_prefill_bwd_workspace_bytes(Nq, Nkv, D, token_slots);
+    // delta is kept in the workspace with lse's indexing: lse must be the dense (batch, head, token) array
+    const int64_t per_b = packed ? token_slots : (int64_t)M * H;
+    if (lse_strides[1] != per_b || lse_strides[0] != (packed ? 0 : (int64_t)Nq * per_b))
+        return fail(BR_ERR_ARG, "lse must be dense: strides (%lld, %lld) expected", (long long)(packed ? 0 : (int64_t)Nq * per_b), (long long)per_b);
+    const size_t need = br_prefill_bwd_workspace_bytes(B, Nq, Nkv, H, D, token_slots);
     if (!workspace || workspace_bytes < need) return fail(BR_ERR_SPACE, "workspace holds %zu bytes, %zu needed", workspace_bytes, need);
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
     BrGeom g;
     int nw;
     make_geom(Nq, Nkv, &g, &nw);
+    if ((long long)M * B * Nkv * ((H + BR_BN - 1) / BR_BN) >= (1LL << 31)) return fail(BR_ERR_ARG, "batch too large for one backward launch");
     BrBwdParams p;
     p.q = q; p.k = k; p.v = v; p.out = out; p.dout = dout; p.plan = plan; p.lse = lse;
     p.lse_b = lse_strides[0]; p.lse_h = lse_strides[1];
     p.dq32 = static_cast<float*>(workspace);
-    p.dk32 = p.dq32 + (size_t)token_slots * Nq * D;
-    p.dv32 = p.dk32 + (size_t)token_slots * Nkv * D;
-    p.acc_b = packed ? 0 : (long long)M * H;
+    p.dk32 = p.dq32 + (size_t)B * Nq * H * D;
+    p.dv32 = p.dk32 + (size_t)B * Nkv * H * D;
+    p.delta = reinterpret_cast<float*>(static_cast<char*>(workspace) + up256((size_t)B * (Nq + 2 * Nkv) * H * D * sizeof(float)));
+    if ((long long)(2 * M - 1) * B * Nkv * ((H + BR_BN - 1) / BR_BN) >= (1LL << 31)) return fail(BR_ERR_ARG, "batch too large for one backward launch");
+    p.dq = dq; p.dk = dk; p.dv = dv;
+    p.dq_b = dq_strides[0]; p.dq_h = dq_strides[1]; p.dq_t = dq_strides[2];
+    p.dk_b = dk_strides[0]; p.dk_h = dk_strides[1]; p.dk_t = dk_strides[2];
+    p.dv_b = dv_strides[0]; p.dv_h = dv_strides[1]; p.dv_t = dv_strides[2];
     p.q32_b = (unsigned)q_strides[0]; p.q32_h = (unsigned)q_strides[1]; p.q32_t = (unsigned)q_strides[2];
     p.k32_b = (unsigned)k_strides[0]; p.k32_h = (unsigned)k_strides[1]; p.k32_t = (unsigned)k_strides[2];
     p.v32_b = (unsigned)v_strides[0]; p.v32_h = (unsigned)v_strides[1]; p.v32_t = (unsigned)v_strides[2];
@@ -402,10 +412,7 @@ int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out,
     p.scale = scale;
     p.scale_log2 = scale * 1.4426950408889634f;
     p.max_items = br_plan_max_items_view0(B, M, H, br_tokens_per_tile(g));
-    const long long sdq[3] = {dq_strides[0], dq_strides[1], dq_strides[2]}, sdk[3] = {dk_strides[0], dk_strides[1], dk_strides[2]},
-                    sdv[3] = {dv_strides[0], dv_strides[1], dv_strides[2]};
-    const int lrc = br_launch_bwd(p, D, nw, n_cu, dq, dk, dv, sdq, sdk, sdv, token_slots, packed ? 0 : (long long)M * H,
-                                  static_cast<hipStream_t>(stream));
+    const int lrc = br_launch_bwd(p, D, nw, n_cu, static_cast<hipStream_t>(stream));
     if (lrc) return fail(BR_ERR_ARG, "no backward kernel for head dim %d with %d query heads per kv head (code %d)", D, g.G, lrc);
     return check_launch("backward launch");
 }

@@ -2,40 +2,38 @@
 //
 // The reference has no hand-written backward: its trainable hooks (blockrank_std_attention.py:96-262, :472-650,
 // used by trainer.py:79-101) are differentiated by torch autograd over dense masked tensors, and its Triton
-// hook refuses (blockrank_triton_kernel_attention.py:759-761).  This kernel computes the same gradients
+// hook refuses (blockrank_triton_kernel_attention.py:759-761).  These kernels compute the same gradients
 //     P = softmax(S),  dV = P^T dO,  dP = dO V^T,  dS = P * (dP - rowsum(dO * O)),
 //     dQ = scale * dS K,  dK = scale * dS^T Q        (dK, dV summed over the query heads of a kv head)
-// over exactly the (query tile, key tile) pairs the forward visits: it walks the forward's own work items
-// (view 0 of the request plan), one workgroup per (item, head group), a wave per 32 rows of one query head.
-// P is rebuilt from the log-sum-exp the forward saved, so an item needs nothing from the items that share
-// its rows (the query block's key walk is split over several).
+// over exactly the (query row, key) pairs the forward visits.  P is rebuilt from the log-sum-exp the forward
+// saved.  Two kernels, so that every sum that has one owner is kept in that owner's registers:
 //
-// Per wave and 64-key tile (K, V tile staged in LDS by the whole workgroup):
-//   S^T = K Q^T, dP^T = V dO^T     accumulators: lane = query row, registers = keys
-//        -> dS^T (bf16) is directly the A operand of   dQ += dS K      (K read with transposing LDS reads)
-//   S = Q K^T, dP = dO V^T         the same products with the operands exchanged: lane = key, registers = rows
-//        -> P, dS (bf16) are directly the A operands of dV += P^T dO,  dK += dS^T Q
-//           (dO and Q as "lane = dim, registers = rows" operands, transposed once per item through LDS)
-// Recomputing S and dP in the second orientation costs 32 of the 112 MFMAs per tile and saves moving P
-// and dS through LDS.
-// dQ stays in registers over the item's walk; dK and dV contributions of a tile leave as fp32 atomic adds
-// into accumulation buffers (several items and the heads of a group add to the same key rows), and so
-// does dQ at the end of the item.  A last kernel converts the three buffers to bf16 tensors.
+//   br_bwd_dq_kernel   query-major: walks the forward's own work items (view 0 of the request plan), one
+//                      workgroup per (item, head group), a wave per 32 rows of one query head.  Per 64-key tile
+//                      (K, V staged in LDS):  S^T = K Q^T, dP^T = V dO^T  (lane = query row, registers = keys)
+//                      -> dS^T in bf16 is directly the A operand of dQ += dS K (K through transposing LDS reads).
+//                      An item that owns its rows stores dQ; the items that share the query block's rows (its key
+//                      walk is split) add into a small fp32 buffer that a finishing kernel converts.  Also writes
+//                      delta = rowsum(dO * O) for the second kernel.
+//   br_bwd_dkv_kernel  key-major: one workgroup per (64-key tile, kv head); a wave owns 32 of the keys and walks,
+//                      for half of the group's query heads, every 32-row block that sees them (the rest of the
+//                      key's own block from the diagonal on; for prefix keys all later blocks; for document keys
+//                      the query block).  S = Q K^T, dP = dO V^T (lane = key, registers = rows) -> P and dS in
+//                      bf16 are directly the A operands of dV += P^T dO and dK += dS^T Q, with dO and Q as
+//                      "lane = dim, registers = rows" operands obtained by transposing LDS reads of the wave's
+//                      own copy of the rows.  dK and dV never leave the registers until the walk ends: no atomics.
 #include "br_common.h"
 
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-
-}  // namespace
-
-
-namespace {
 
 __device__ inline uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ inline bf16x8 as_bf16x8(uint4 u) {
@@ -60,12 +58,11 @@ __device__ inline bf16x8 pack8(const f32x16& x, int s) {
 
 template <int D>
 struct Bwd {
-    static constexpr int RS = 2 * D + 16;          // LDS row stride in bytes (16 bytes of padding spread the banks)
+    static constexpr int RS = 2 * D + 32;          // LDS row stride in bytes: the 32 bytes of padding put the four rows of a transposing read in different banks
     static constexpr int CPR = D / 8;              // 16-byte pieces per row
     static constexpr int NC = D / 16, ND = D / 32;
     static constexpr int tileBytes = BR_BN * RS;
-    static constexpr int waveBytes = BR_RB * RS;
-    static constexpr int ldsBytes(int nw) { return 2 * tileBytes + nw * waveBytes; }
+    static constexpr int rowsBytes = BR_RB * RS;
 
     // Row (r0 + lane % 32), dims 16c + 8 * (lane / 32) .. +7 of a row-major LDS tile: the operand layout of a
     // product that contracts over the head dim.
@@ -86,7 +83,12 @@ struct Bwd {
         return a.b8;
     }
 
-    static __device__ void run_item(const BrBwdParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem, int NW) {
+    // ---------------------------------------------------------------------------------------------------------
+    // dQ (and delta) of one work item
+    // ---------------------------------------------------------------------------------------------------------
+    static constexpr int dqLdsBytes = 2 * tileBytes;
+
+    static __device__ __forceinline__ void dq_item(const BrBwdParams& p, const BrPlanView& pv, const BrItem& it, int hg, char* smem, int NW) {
         const int tid = threadIdx.x, NT = NW * 64;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
         const BrGeom& ge = p.geom;
@@ -102,16 +104,12 @@ struct Bwd {
         const int qtok0 = it.tok_m;
         char* Ks = smem;
         char* Vs = smem + tileBytes;
-        char* Ws = smem + 2 * tileBytes + wave * waveBytes;
         const char* kbase = reinterpret_cast<const char*>(p.k) + 2 * ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh);
         const char* vbase = reinterpret_cast<const char*>(p.v) + 2 * ((unsigned long long)p.v32_b * (unsigned)b + (unsigned long long)p.v32_h * (unsigned)kvh);
 
-        // ---- per item: Q and dO of this wave's rows in both operand layouts, the rows' log-sum-exp and
-        // delta = rowsum(dO * O) ----
-        bf16x8 qf[NC], dof[NC];        // lane = row, registers = dims
-        bf16x8 qt[ND][2], dot[ND][2];  // lane = dim, registers = rows
-        float lse_l = 0.f, delta_l = 0.f;          // of row row0 + ln
-        float lse_r[16], delta_r[16];              // of row row0 + 8 (v / 4) + 4 lh + v % 4
+        // Q and dO of this wave's rows (lane = row, registers = dims), the rows' log-sum-exp and delta
+        bf16x8 qf[NC], dof[NC];
+        float lse_l = 0.f, delta_l = 0.f;
         if (rb_active) {
             const int last = len_m - 1 - row0;
             const int r = ln < last ? ln : last;       // rows past the block's end repeat its last row; they are masked below
@@ -132,50 +130,24 @@ struct Bwd {
                 for (int e = 0; e < 8; ++e) dsum += (float)o8[e] * (float)dof[c][e];
             }
             delta_l = dsum + __shfl_xor(dsum, 32);
-            lse_l = p.lse[(long long)b * p.lse_b + (long long)head * p.lse_h + tok];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int i = 8 * (v >> 2) + 4 * lh + (v & 3);
-                lse_r[v] = __shfl(lse_l, i);
-                delta_r[v] = __shfl(delta_l, i);
-            }
-            // transposed operands through the wave's own LDS rows (a wave's LDS operations complete in order)
-#pragma unroll
-            for (int c = 0; c < NC; ++c) *reinterpret_cast<bf16x8*>(Ws + ln * RS + c * 32 + lh * 16) = qf[c];
-            __threadfence_block();
-#pragma unroll
-            for (int db = 0; db < ND; ++db)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) qt[db][s] = read_col(Ws, 16 * s, db, lane);
-            __threadfence_block();
-#pragma unroll
-            for (int c = 0; c < NC; ++c) *reinterpret_cast<bf16x8*>(Ws + ln * RS + c * 32 + lh * 16) = dof[c];
-            __threadfence_block();
-#pragma unroll
-            for (int db = 0; db < ND; ++db)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) dot[db][s] = read_col(Ws, 16 * s, db, lane);
+            const long long li = (long long)b * p.lse_b + (long long)head * p.lse_h + tok;
+            lse_l = p.lse[li];
+            // every item of a row block computes the same delta; the one that starts the key walk publishes it
+            if (it.f_lo == 0 && lh == 0 && ln <= last) p.delta[li] = delta_l;
         } else {
 #pragma unroll
             for (int c = 0; c < NC; ++c) qf[c] = dof[c] = as_bf16x8(uint4{0u, 0u, 0u, 0u});
-#pragma unroll
-            for (int db = 0; db < ND; ++db)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) qt[db][s] = dot[db][s] = as_bf16x8(uint4{0u, 0u, 0u, 0u});
-#pragma unroll
-            for (int v = 0; v < 16; ++v) lse_r[v] = delta_r[v] = 0.f;
         }
 
         f32x16 dq[ND];
 #pragma unroll
         for (int db = 0; db < ND; ++db) dq[db] = zero16();
 
-        // ---- the item's key walk: the earlier blocks' tiles it covers, then its own block's up to the diagonal ----
+        // the item's key walk: the earlier blocks' tiles it covers, then its own block's up to the diagonal
         const int2* tiles_b = pv.tiles + (size_t)b * pv.tps;
         const bool table = it.pe > 1;
         const int nprev = it.nprev;
         const int f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
-        const long long slot_b = (long long)b * p.acc_b;
         for (int f = it.f_lo; f < f_end; ++f) {
             const bool self = f >= nprev;
             int tok0, nvalid, key0 = 0;
@@ -218,94 +190,327 @@ struct Bwd {
             }
             if (!rb_active) nkb = 0;
             for (int kb = 0; kb < nkb; ++kb) {
-                // -- lane = query row: dS^T, then dQ += dS K --
-                {
-                    f32x16 st = zero16(), dpt = zero16();
+                f32x16 st = zero16(), dpt = zero16();
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) {
-                        st = mma(read_row(Ks, kb * 32, c, ln, lh), qf[c], st);
-                        dpt = mma(read_row(Vs, kb * 32, c, ln, lh), dof[c], dpt);
-                    }
-                    const int lim_c = self ? row0 + ln - key0 + 1 : BR_BN;                 // keys [0, lim) of the tile are visible
-                    int lim = nvalid < lim_c ? nvalid : lim_c;
-                    if (row0 + ln >= len_m) lim = 0;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int key = kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                        const float pr = __builtin_amdgcn_exp2f(st[v] * p.scale_log2 - lse_l);
-                        st[v] = key < lim ? pr * (dpt[v] - delta_l) * p.scale : 0.f;
-                    }
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        const bf16x8 a = pack8(st, s);
-#pragma unroll
-                        for (int db = 0; db < ND; ++db) dq[db] = mma(a, read_col(Ks, kb * 32 + 16 * s, db, lane), dq[db]);
-                    }
+                for (int c = 0; c < NC; ++c) {
+                    st = mma(read_row(Ks, kb * 32, c, ln, lh), qf[c], st);
+                    dpt = mma(read_row(Vs, kb * 32, c, ln, lh), dof[c], dpt);
                 }
-                // -- lane = key: P and dS, then dV += P^T dO and dK += dS^T Q for this half's 32 keys --
-                {
-                    f32x16 sn = zero16(), dpn = zero16();
+                // K as "lane = dim" operand: the transposing reads are issued ahead of the arithmetic that hides them
+                bf16x8 kc[2][ND];
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) {
-                        sn = mma(qf[c], read_row(Ks, kb * 32, c, ln, lh), sn);
-                        dpn = mma(dof[c], read_row(Vs, kb * 32, c, ln, lh), dpn);
-                    }
-                    const int key = kb * 32 + ln;
-                    const bool key_ok = key < nvalid;
+                for (int s = 0; s < 2; ++s)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int row = row0 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                        const bool vis = key_ok && row < len_m && (!self || key0 + key <= row);
-                        const float pr = vis ? __builtin_amdgcn_exp2f(sn[v] * p.scale_log2 - lse_r[v]) : 0.f;
-                        sn[v] = pr;
-                        dpn[v] = vis ? pr * (dpn[v] - delta_r[v]) * p.scale : 0.f;
-                    }
-                    const bf16x8 p0 = pack8(sn, 0), p1 = pack8(sn, 1), d0 = pack8(dpn, 0), d1 = pack8(dpn, 1);
-                    // accumulator: lane = dim 32 db + ln, register v = key kb*32 + 8 (v/4) + 4 lh + v%4
-                    const long long rowk = slot_b + tok0 + kb * 32 + 4 * lh;
+                    for (int db = 0; db < ND; ++db) kc[s][db] = read_col(Ks, kb * 32 + 16 * s, db, lane);
+                const int lim_c = self ? row0 + ln - key0 + 1 : BR_BN;                 // keys [0, lim) of the tile are visible
+                int lim = nvalid < lim_c ? nvalid : lim_c;
+                if (row0 + ln >= len_m) lim = 0;
 #pragma unroll
-                    for (int db = 0; db < ND; ++db) {
-                        f32x16 av = mma(p0, dot[db][0], zero16());
-                        av = mma(p1, dot[db][1], av);
-                        f32x16 ak = mma(d0, qt[db][0], zero16());
-                        ak = mma(d1, qt[db][1], ak);
-                        float* dvp = p.dv32 + (rowk * p.Nkv + kvh) * D + db * 32 + ln;
-                        float* dkp = p.dk32 + (rowk * p.Nkv + kvh) * D + db * 32 + ln;
+                for (int v = 0; v < 16; ++v) {
+                    const int key = kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                    // hidden pairs get exponent -inf, i.e. probability 0, without a branch (every operand is finite)
+                    const float pr = __builtin_amdgcn_exp2f(key < lim ? st[v] * p.scale_log2 - lse_l : -INFINITY);
+                    st[v] = pr * (dpt[v] - delta_l) * p.scale;
+                }
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int kr = 8 * (v >> 2) + (v & 3);                       // key row minus 4 lh
-                            if (kb * 32 + 4 * lh + kr < nvalid) {
-                                unsafeAtomicAdd(dvp + (long long)kr * p.Nkv * D, av[v]);
-                                unsafeAtomicAdd(dkp + (long long)kr * p.Nkv * D, ak[v]);
-                            }
-                        }
-                    }
+                for (int s = 0; s < 2; ++s) {
+                    const bf16x8 a = pack8(st, s);
+#pragma unroll
+                    for (int db = 0; db < ND; ++db) dq[db] = mma(a, kc[s][db], dq[db]);
                 }
             }
         }
-        // ---- dQ of this wave's rows: lane = dim 32 db + ln, register v = row 8 (v/4) + 4 lh + v%4 ----
-        if (rb_active) {
-            float* dqp = p.dq32 + ((slot_b + qtok0 + row0 + 4 * lh) * p.Nq + head) * D + ln;
+        // dQ of this wave's rows: lane = dim 32 db + ln, register v = row 8 (v/4) + 4 lh + v%4
+        if (!rb_active) return;
+        if (it.slot < 0) {
+            __bf16* dst = reinterpret_cast<__bf16*>(p.dq) + (long long)b * p.dq_b + (long long)head * p.dq_h +
+                          (long long)(qtok0 + row0 + 4 * lh) * p.dq_t + ln;
 #pragma unroll
             for (int db = 0; db < ND; ++db)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int r = 8 * (v >> 2) + (v & 3);
-                    if (row0 + 4 * lh + r < len_m) unsafeAtomicAdd(dqp + (long long)r * p.Nq * D + db * 32, dq[db][v]);
+                    if (row0 + 4 * lh + r < len_m) dst[(long long)r * p.dq_t + db * 32] = (__bf16)dq[db][v];
+                }
+        } else {
+            // shared rows (the query block): [b][head][row of the block][D] fp32
+            float* dqp = p.dq32 + (((long long)b * p.Nq + head) * p.H + row0 + 4 * lh) * D + ln;
+#pragma unroll
+            for (int db = 0; db < ND; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = 8 * (v >> 2) + (v & 3);
+                    if (row0 + 4 * lh + r < len_m) unsafeAtomicAdd(dqp + r * D + db * 32, dq[db][v]);
                 }
         }
+    }
+
+    // ---------------------------------------------------------------------------------------------------------
+    // dK, dV of one 64-key tile of one kv head.  256 threads: wave = (key half kb, head parity hsel).
+    // ---------------------------------------------------------------------------------------------------------
+    static constexpr int dkvLdsBytes = 4 * (2 * rowsBytes + 256);     // per wave: its copy of 32 rows of Q and of dO, their lse and delta
+
+    // mq_only < 0: the tile's main workgroup - viewers are the rest of the keys' own block and, for document keys,
+    // the query block; mq_only >= 1 (prefix keys only): the rows of block mq_only.  Prefix keys have a workgroup
+    // per viewing block, so their sums meet in fp32 buffers (atomic adds); all other keys have one owner, which
+    // stores bf16.
+    static __device__ __forceinline__ void dkv_tile(const BrBwdParams& p, const BrPlanView& pv, int b, int m, int kt, int kvh, int mq_only, char* smem) {
+        const int tid = threadIdx.x;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
+        const int kb = wave & 1, hsel = wave >> 1;
+        const int G = p.geom.G, M = p.M;
+        const int len_m = pv.len[b * M + m], tok_m = pv.tok[b * M + m];
+        const int key0 = kt * BR_BN;
+        const int nvalid = len_m - key0 < BR_BN ? len_m - key0 : BR_BN;      // > 0: checked by the caller
+        char* Wq = smem + wave * (2 * rowsBytes + 256);
+        char* Wd = Wq + rowsBytes;
+        float* Wl = reinterpret_cast<float*>(Wd + rowsBytes);       // [32] log-sum-exp, [32] delta
+
+        // this wave's 32 keys as operands (lane = key, registers = dims); rows past the real keys are zero
+        bf16x8 kf[NC], vf[NC];
+        {
+            const int key = kb * 32 + ln;
+            const bool on = key < nvalid;
+            const unsigned tok = (unsigned)(tok_m + key0 + (on ? key : 0));
+            const char* krow = reinterpret_cast<const char*>(p.k) +
+                               2 * ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh + (unsigned long long)p.k32_t * tok);
+            const char* vrow = reinterpret_cast<const char*>(p.v) +
+                               2 * ((unsigned long long)p.v32_b * (unsigned)b + (unsigned long long)p.v32_h * (unsigned)kvh + (unsigned long long)p.v32_t * tok);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                kf[c] = as_bf16x8(on ? ld16(krow + c * 32 + lh * 16) : uint4{0u, 0u, 0u, 0u});
+                vf[c] = as_bf16x8(on ? ld16(vrow + c * 32 + lh * 16) : uint4{0u, 0u, 0u, 0u});
+            }
+        }
+        f32x16 dk[ND], dv[ND];      // lane = dim 32 db + ln, register v = key kb*32 + 8 (v/4) + 4 lh + v%4
+#pragma unroll
+        for (int db = 0; db < ND; ++db) dk[db] = dv[db] = zero16();
+        const bool half_on = kb * 32 < nvalid;
+
+        // The wave's steps: (32-row block that sees these keys, one of the wave's heads).  Row blocks come from up to
+        // two blocks: the keys' own block from the diagonal on, then the query block (document keys) - or, for a
+        // prefix-key workgroup of a viewing block, that block alone.  Every quantity below is wave-uniform.
+        struct Step {
+            int r0, nrows, tok, head, self;
+        };
+        const int blk0 = mq_only < 0 ? m : mq_only;
+        const int blk1 = (mq_only < 0 && m > 0 && m < M - 1) ? M - 1 : -1;
+        int seg = (half_on && hsel < G) ? 0 : 2;               // 2 = exhausted
+        int cur_blk = blk0, cur_len = pv.len[b * M + blk0], cur_tok = pv.tok[b * M + blk0];
+        int rb = mq_only < 0 ? key0 / BR_RB : 0, hl = hsel;
+        auto next_step = [&](Step& st) -> bool {
+            while (seg < 2) {
+                if (rb * BR_RB >= cur_len) {
+                    seg = (seg == 0 && blk1 >= 0) ? 1 : 2;
+                    if (seg == 1) {
+                        cur_blk = blk1;
+                        cur_len = pv.len[b * M + blk1];
+                        cur_tok = pv.tok[b * M + blk1];
+                        rb = 0;
+                    }
+                    continue;
+                }
+                const int r0 = rb * BR_RB;
+                const int nrows = cur_len - r0 < BR_RB ? cur_len - r0 : BR_RB;
+                const int self = cur_blk == m;
+                // causal rule on the block's own keys: nothing to do if even the last row precedes this half's first key
+                if (self && r0 + nrows - 1 < key0 + kb * 32) {
+                    ++rb;
+                    continue;
+                }
+                st.r0 = r0; st.nrows = nrows; st.tok = cur_tok + r0; st.head = kvh * G + hl; st.self = self;
+                hl += 2;
+                if (hl >= G) {
+                    hl = hsel;
+                    ++rb;
+                }
+                return true;
+            }
+            return false;
+        };
+        // Q and dO rows of a step (lane = row, registers = dims; rows past the block's end repeat its last row and
+        // are masked later), and the rows' log-sum-exp and delta (lane ln holds row ln's)
+        auto load_step = [&](const Step& st, uint4 (&qv)[NC], uint4 (&gv)[NC], float& lse_l, float& delta_l) {
+            const int r = ln < st.nrows ? ln : st.nrows - 1;
+            const unsigned tok = (unsigned)(st.tok + r);
+            const char* qrow = reinterpret_cast<const char*>(p.q) +
+                               2 * ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)st.head + (unsigned long long)p.q32_t * tok);
+            const char* grow = reinterpret_cast<const char*>(p.dout) +
+                               2 * ((unsigned long long)p.g32_b * (unsigned)b + (unsigned long long)p.g32_h * (unsigned)st.head + (unsigned long long)p.g32_t * tok);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                qv[c] = ld16(qrow + c * 32 + lh * 16);
+                gv[c] = ld16(grow + c * 32 + lh * 16);
+            }
+            const long long li = (long long)b * p.lse_b + (long long)st.head * p.lse_h + tok;
+            lse_l = p.lse[li];
+            delta_l = p.delta[li];
+        };
+        {
+            // Per step: copy the rows into the wave's LDS area, S = Q K^T and dP = dO V^T from the registers - after
+            // which the registers are free, so the next step's loads are issued into them and fly while the rest of
+            // this step (softmax terms, dV and dK products, which read the LDS copy) is computed.
+            Step cur, nxt;
+            uint4 qv[NC], gv[NC];
+            float lse_c = 0.f, delta_c = 0.f, lse_n = 0.f, delta_n = 0.f;
+            bool have = next_step(cur);
+            if (have) load_step(cur, qv, gv, lse_c, delta_c);
+            while (have) {
+                const bool have_next = next_step(nxt);
+                // (a wave's LDS operations complete in order; the empty asm stops the compiler from reordering them)
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    *reinterpret_cast<uint4*>(Wq + ln * RS + c * 32 + lh * 16) = qv[c];
+                    *reinterpret_cast<uint4*>(Wd + ln * RS + c * 32 + lh * 16) = gv[c];
+                }
+                if (lh == 0) {
+                    Wl[ln] = lse_c;
+                    Wl[32 + ln] = delta_c;
+                }
+                asm volatile("" ::: "memory");
+                f32x16 sn = zero16(), dpn = zero16();
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    sn = mma(as_bf16x8(qv[c]), kf[c], sn);
+                    dpn = mma(as_bf16x8(gv[c]), vf[c], dpn);
+                }
+                if (have_next) load_step(nxt, qv, gv, lse_n, delta_n);
+                // the "lane = dim" operands: all transposing reads are issued here, ahead of the arithmetic that hides
+                // their latency (the compiler keeps each such read next to its use)
+                bf16x8 cd[ND][2], cq[ND][2];
+#pragma unroll
+                for (int db = 0; db < ND; ++db)
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; ++s2) {
+                        cd[db][s2] = read_col(Wd, 16 * s2, db, lane);
+                        cq[db][s2] = read_col(Wq, 16 * s2, db, lane);
+                    }
+                const int key = kb * 32 + ln;
+                const bool key_ok = key < nvalid;
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) {
+                    // accumulator registers 4 v4 .. 4 v4 + 3 hold rows r0 + 8 v4 + 4 lh + 0..3
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(Wl + 8 * v4 + 4 * lh);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(Wl + 32 + 8 * v4 + 4 * lh);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int v = 4 * v4 + e, i = 8 * v4 + 4 * lh + e;
+                        // hidden pairs get exponent -inf, i.e. probability 0, without a branch (every operand is finite)
+                        const bool vis = key_ok && i < cur.nrows && (!cur.self || key0 + key <= cur.r0 + i);
+                        const float pr = __builtin_amdgcn_exp2f(vis ? sn[v] * p.scale_log2 - l4[e] : -INFINITY);
+                        sn[v] = pr;
+                        dpn[v] = pr * (dpn[v] - d4[e]) * p.scale;
+                    }
+                }
+                const bf16x8 p0 = pack8(sn, 0), p1 = pack8(sn, 1), d0 = pack8(dpn, 0), d1 = pack8(dpn, 1);
+#pragma unroll
+                for (int db = 0; db < ND; ++db) {
+                    dv[db] = mma(p0, cd[db][0], dv[db]);
+                    dk[db] = mma(d0, cq[db][0], dk[db]);
+                }
+#pragma unroll
+                for (int db = 0; db < ND; ++db) {
+                    dv[db] = mma(p1, cd[db][1], dv[db]);
+                    dk[db] = mma(d1, cq[db][1], dk[db]);
+                }
+                cur = nxt;
+                lse_c = lse_n;
+                delta_c = delta_n;
+                have = have_next;
+            }
+        }
+
+        if (m == 0 && M > 1) {
+            // prefix keys: add into the fp32 buffers [b][kv head][key][D]
+            float* k32 = p.dk32 + (((long long)b * p.Nkv + kvh) * p.H + key0 + kb * 32 + 4 * lh) * D + ln;
+            float* v32 = p.dv32 + (((long long)b * p.Nkv + kvh) * p.H + key0 + kb * 32 + 4 * lh) * D + ln;
+            if (half_on) {
+#pragma unroll
+                for (int db = 0; db < ND; ++db)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int kr = 8 * (v >> 2) + (v & 3);
+                        if (kb * 32 + 4 * lh + kr < nvalid) {
+                            unsafeAtomicAdd(k32 + kr * D + db * 32, dk[db][v]);
+                            unsafeAtomicAdd(v32 + kr * D + db * 32, dv[db][v]);
+                        }
+                    }
+            }
+            return;
+        }
+        // sum the two head parities of each key half through LDS (dK, then dV), then store bf16
+        float* red = reinterpret_cast<float*>(smem);               // [2 halves][32 keys][D] fp32 = 2 * 32 * D * 4 bytes
+        static_assert(2 * 32 * D * 4 <= dkvLdsBytes, "reduction buffer must fit the waves' row copies");
+        auto reduce_store = [&](f32x16 (&acc)[ND], void* out, long long s_b, long long s_h, long long s_t) {
+            __syncthreads();
+            if (hsel == 1) {
+#pragma unroll
+                for (int db = 0; db < ND; ++db)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) red[(kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3)) * D + db * 32 + ln] = acc[db][v];
+            }
+            __syncthreads();
+            if (hsel == 0) {
+                __bf16* dst = reinterpret_cast<__bf16*>(out) + (long long)b * s_b + (long long)kvh * s_h +
+                              (long long)(tok_m + key0 + kb * 32 + 4 * lh) * s_t + ln;
+#pragma unroll
+                for (int db = 0; db < ND; ++db)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int kr = 8 * (v >> 2) + (v & 3);
+                        const float x = acc[db][v] + red[(kb * 32 + 4 * lh + kr) * D + db * 32 + ln];
+                        if (kb * 32 + 4 * lh + kr < nvalid) dst[(long long)kr * s_t + db * 32] = (__bf16)x;
+                    }
+            }
+        };
+        reduce_store(dk, p.dk, p.dk_b, p.dk_h, p.dk_t);
+        reduce_store(dv, p.dv, p.dv_b, p.dv_h, p.dv_t);
     }
 };
 
 template <int D, int MAXW>
-__global__ __launch_bounds__(MAXW * 64, 1) void br_bwd_kernel(BrBwdParams p) {
+__global__ __launch_bounds__(MAXW * 64, MAXW <= 4 ? 2 : 1) void br_bwd_dq_kernel(BrBwdParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const BrGeom& ge = p.geom;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
     const int item = blockIdx.x / ge.NHG, hg = blockIdx.x - item * ge.NHG;
     if (item >= pv.hdr[BR_PH_QOFF2 + BR_GLOBAL_QUEUE]) return;      // view 0's items come first in the array; view 1 starts here
     const BrItem it = pv.items[item];
-    Bwd<D>::run_item(p, pv, it, hg, smem, blockDim.x >> 6);
+    Bwd<D>::dq_item(p, pv, it, hg, smem, blockDim.x >> 6);
+}
+
+// blockIdx.x enumerates (unit, sequence b, kv head, key tile): units 0 .. M-1 are the blocks' main workgroups, units
+// M .. 2M-2 the workgroups that take the rows of blocks 1 .. M-1 to the prefix keys.
+template <int D>
+__global__ __launch_bounds__(256, 1) void br_bwd_dkv_kernel(BrBwdParams p) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
+    const int KT = (p.H + BR_BN - 1) / BR_BN;
+    int idx = blockIdx.x;
+    const int kt = idx % KT;
+    idx /= KT;
+    const int kvh = idx % p.Nkv;
+    idx /= p.Nkv;
+    const int b = idx % p.B, unit = idx / p.B;
+    const int m = unit < p.M ? unit : 0, mq_only = unit < p.M ? -1 : unit - p.M + 1;
+    const int len_m = pv.len[b * p.M + m];
+    // padded slots of this block (dk and dv of this kv head): zeros, written by the block's first workgroup
+    if (kt == 0 && mq_only < 0 && !pv.hdr[BR_PH_PACKED]) {
+        const int st = pv.start[b * p.M + m], npad = p.H - len_m;
+        constexpr int CP8 = D / 8;
+        const uint4 z = {0u, 0u, 0u, 0u};
+        __bf16* kb_ = reinterpret_cast<__bf16*>(p.dk) + (long long)b * p.dk_b + (long long)kvh * p.dk_h;
+        __bf16* vb_ = reinterpret_cast<__bf16*>(p.dv) + (long long)b * p.dv_b + (long long)kvh * p.dv_h;
+        for (int i = threadIdx.x; i < npad * CP8; i += blockDim.x) {
+            const int r = i / CP8, c8 = i - r * CP8;
+            const long long pos = (long long)m * p.H + (r < st ? r : r + len_m);
+            *reinterpret_cast<uint4*>(kb_ + pos * p.dk_t + c8 * 8) = z;
+            *reinterpret_cast<uint4*>(vb_ + pos * p.dv_t + c8 * 8) = z;
+        }
+    }
+    if (kt * BR_BN >= len_m) return;
+    Bwd<D>::dkv_tile(p, pv, b, m, kt, kvh, mq_only, smem);
 }
 
 __global__ __launch_bounds__(256) void br_fill_zero_kernel(uint4* p, size_t n16) {
@@ -313,59 +518,100 @@ __global__ __launch_bounds__(256) void br_fill_zero_kernel(uint4* p, size_t n16)
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = z;
 }
 
-// fp32 accumulation buffer [slot][heads][D] -> bf16 tensor with (batch, head, token) strides; slots of padded
-// tokens were never added to and come out as zeros.
-__global__ __launch_bounds__(256) void br_bwd_store_kernel(const float* acc, __bf16* dst, long long n_slots, long long slots_per_b, int heads,
-                                                           int D, long long s_b, long long s_h, long long s_t) {
-    const int c4 = D / 4;
-    const long long n = n_slots * heads * c4;
+// dQ of the rows whose key walk was split (the plan's combine list names their query tiles): fp32 sums -> bf16;
+// and zeros for the padded slots of dq.
+template <int D>
+__global__ __launch_bounds__(256) void br_bwd_dq_finish_kernel(BrBwdParams p) {
+    const BrGeom& ge = p.geom;
+    const int T = ge.tpb * BR_RB;
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, T);
+    constexpr int C4 = D / 4;
+    const int m = p.M - 1;
+    const long long n = (long long)pv.hdr[BR_PH_NCOMB] * p.Nq * T * C4;
     for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
-        const long long row = i / c4;
-        const int c = (int)(i - row * c4);
-        const long long slot = row / heads;
-        const int h = (int)(row - slot * heads);
-        const long long b = slots_per_b > 0 ? slot / slots_per_b : 0, t = slots_per_b > 0 ? slot - b * slots_per_b : slot;
-        const float4 x = *reinterpret_cast<const float4*>(acc + row * D + c * 4);
-        typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-        typedef float f32x4 __attribute__((ext_vector_type(4)));
-        const f32x4 f = {x.x, x.y, x.z, x.w};
-        *reinterpret_cast<bf16x4*>(dst + b * s_b + h * s_h + t * s_t + c * 4) = __builtin_convertvector(f, bf16x4);
+        const int c = (int)(i % C4);
+        long long r = i / C4;
+        const int row_in = (int)(r % T);
+        r /= T;
+        const int head = (int)(r % p.Nq), ci = (int)(r / p.Nq);
+        const BrComb cb = pv.comb[ci];
+        const int row = cb.t0 + row_in;
+        if (row >= pv.len[cb.b * p.M + m]) continue;
+        const f32x4 x = *reinterpret_cast<const f32x4*>(p.dq32 + (((long long)cb.b * p.Nq + head) * p.H + row) * D + c * 4);
+        __bf16* dst = reinterpret_cast<__bf16*>(p.dq) + (long long)cb.b * p.dq_b + (long long)head * p.dq_h +
+                      (long long)(pv.tok[cb.b * p.M + m] + row) * p.dq_t + c * 4;
+        *reinterpret_cast<bf16x4*>(dst) = __builtin_convertvector(x, bf16x4);
+    }
+    // dK, dV of the prefix keys (summed over the workgroups of every viewing block)
+    if (p.M > 1) {
+        const long long nk = (long long)p.B * p.Nkv * p.H * C4;
+        for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < nk; i += (long long)gridDim.x * blockDim.x) {
+            const int c = (int)(i % C4);
+            long long r = i / C4;
+            const int key = (int)(r % p.H);
+            r /= p.H;
+            const int kvh = (int)(r % p.Nkv), b = (int)(r / p.Nkv);
+            if (key >= pv.len[b * p.M]) continue;
+            const long long src = (((long long)b * p.Nkv + kvh) * p.H + key) * D + c * 4;
+            const long long tokk = pv.tok[b * p.M] + key;
+            *reinterpret_cast<bf16x4*>(reinterpret_cast<__bf16*>(p.dk) + (long long)b * p.dk_b + (long long)kvh * p.dk_h + tokk * p.dk_t + c * 4) =
+                __builtin_convertvector(*reinterpret_cast<const f32x4*>(p.dk32 + src), bf16x4);
+            *reinterpret_cast<bf16x4*>(reinterpret_cast<__bf16*>(p.dv) + (long long)b * p.dv_b + (long long)kvh * p.dv_h + tokk * p.dv_t + c * 4) =
+                __builtin_convertvector(*reinterpret_cast<const f32x4*>(p.dv32 + src), bf16x4);
+        }
+    }
+    if (pv.hdr[BR_PH_PACKED]) return;
+    constexpr int CP8 = D / 8;
+    const uint4 z = {0u, 0u, 0u, 0u};
+    for (int w = blockIdx.x; w < p.B * p.M * p.Nq; w += gridDim.x) {
+        const int bm = w / p.Nq, head = w - bm * p.Nq;
+        const int b = bm / p.M, mm = bm - b * p.M;
+        const int st = pv.start[bm], ln = pv.len[bm], npad = p.H - ln;
+        __bf16* base = reinterpret_cast<__bf16*>(p.dq) + (long long)b * p.dq_b + (long long)head * p.dq_h;
+        for (int idx = threadIdx.x; idx < npad * CP8; idx += blockDim.x) {
+            const int r = idx / CP8, c8 = idx - r * CP8;
+            const long long pos = (long long)mm * p.H + (r < st ? r : r + ln);
+            *reinterpret_cast<uint4*>(base + pos * p.dq_t + c8 * 8) = z;
+        }
     }
 }
 
 template <int D, int MAXW>
-int launch_bwd(const BrBwdParams& p, int NW, hipStream_t stream) {
-    const int lds = Bwd<D>::ldsBytes(NW);
-    static int armed = 0;          // largest dynamic LDS size this instance has been enabled for
-    if (lds > armed) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&br_bwd_kernel<D, MAXW>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+int launch_dq(const BrBwdParams& p, int NW, hipStream_t stream) {
+    const int lds = Bwd<D>::dqLdsBytes;
+    static bool armed = false;
+    if (!armed) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&br_bwd_dq_kernel<D, MAXW>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return -2;
-        armed = lds;
+        armed = true;
     }
-    hipLaunchKernelGGL((br_bwd_kernel<D, MAXW>), dim3(p.max_items * p.geom.NHG), dim3(NW * 64), lds, stream, p);
+    hipLaunchKernelGGL((br_bwd_dq_kernel<D, MAXW>), dim3(p.max_items * p.geom.NHG), dim3(NW * 64), lds, stream, p);
+    return 0;
+}
+
+template <int D>
+int launch_all(const BrBwdParams& p, int NW, int n_cu, hipStream_t stream) {
+    const size_t n16 = (size_t)p.B * (p.Nq + 2 * p.Nkv) * p.H * D / 4;      // dq32, dk32, dv32 are contiguous
+    hipLaunchKernelGGL(br_fill_zero_kernel, dim3(n_cu * 4), dim3(256), 0, stream, reinterpret_cast<uint4*>(p.dq32), n16);
+    const int rc = NW <= 4 ? launch_dq<D, 4>(p, NW, stream) : launch_dq<D, 8>(p, NW, stream);
+    if (rc) return rc;
+    const int lds = Bwd<D>::dkvLdsBytes;
+    static bool armed = false;
+    if (!armed) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&br_bwd_dkv_kernel<D>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
+        armed = true;
+    }
+    const int KT = (p.H + BR_BN - 1) / BR_BN;
+    hipLaunchKernelGGL((br_bwd_dkv_kernel<D>), dim3((2 * p.M - 1) * p.B * p.Nkv * KT), dim3(256), lds, stream, p);
+    hipLaunchKernelGGL((br_bwd_dq_finish_kernel<D>), dim3(n_cu * 4), dim3(256), 0, stream, p);
     return 0;
 }
 
 }  // namespace
 
-// dq/dk/dv: bf16 tensors with (batch, head, token) element strides.  n_slots = token slots in total
-// (B * M * H padded, or the packed token count), slots_per_b = M * H for a padded layout, 0 for a packed one.
-// Returns 0 on success, -1 if D has no instance, -2 if the kernel's LDS size could not be set.
-int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, void* dq, void* dk, void* dv, const long long* sdq, const long long* sdk,
-                  const long long* sdv, long long n_slots, long long slots_per_b, hipStream_t stream) {
-    const size_t n16 = (size_t)n_slots * (p.Nq + 2 * p.Nkv) * D / 4;          // the three buffers are contiguous
-    hipLaunchKernelGGL(br_fill_zero_kernel, dim3(n_cu * 8), dim3(256), 0, stream, reinterpret_cast<uint4*>(p.dq32), n16);
-    int rc;
-    if (D == 128) rc = NW <= 4 ? launch_bwd<128, 4>(p, NW, stream) : launch_bwd<128, 8>(p, NW, stream);
-    else if (D == 64) rc = NW <= 4 ? launch_bwd<64, 4>(p, NW, stream) : launch_bwd<64, 8>(p, NW, stream);
-    else return -1;
-    if (rc) return rc;
-    const int grid = n_cu * 8;
-    hipLaunchKernelGGL(br_bwd_store_kernel, dim3(grid), dim3(256), 0, stream, p.dq32, static_cast<__bf16*>(dq), n_slots, slots_per_b, p.Nq, D,
-                       sdq[0], sdq[1], sdq[2]);
-    hipLaunchKernelGGL(br_bwd_store_kernel, dim3(grid), dim3(256), 0, stream, p.dk32, static_cast<__bf16*>(dk), n_slots, slots_per_b, p.Nkv, D,
-                       sdk[0], sdk[1], sdk[2]);
-    hipLaunchKernelGGL(br_bwd_store_kernel, dim3(grid), dim3(256), 0, stream, p.dv32, static_cast<__bf16*>(dv), n_slots, slots_per_b, p.Nkv, D,
-                       sdv[0], sdv[1], sdv[2]);
-    return 0;
+// Returns 0 on success, -1 if D has no instance, -2 if a kernel's LDS size could not be set.
+int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, hipStream_t stream) {
+    if (D == 128) return launch_all<128>(p, NW, n_cu, stream);
+    if (D == 64) return launch_all<64>(p, NW, n_cu, stream);
+    return -1;
 }

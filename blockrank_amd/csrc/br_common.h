@@ -294,7 +294,7 @@ struct BrPrefillParams {
     long long lse_b, lse_h;
 };
 
-// Arguments of the backward kernel (bf16).
+// Arguments of the backward kernels (bf16).
 struct BrBwdParams {
     const void* q;
     const void* k;
@@ -303,11 +303,15 @@ struct BrBwdParams {
     const void* dout;
     const int* plan;
     const float* lse;          // base-2 log-sum-exp of every real row, as the forward wrote it
+    float* delta;              // rowsum(dO * O) of every real row, same indexing as lse (written by the dQ kernel)
     long long lse_b, lse_h;
-    float* dq32;               // [slot][Nq][D] fp32, slot = b * acc_b + token
-    float* dk32;               // [slot][Nkv][D]
+    float* dq32;               // [B][Nq][H][D] fp32: dQ sums of the query block's rows when several items share them
+    float* dk32;               // [B][Nkv][H][D] fp32: dK, dV sums of the prefix keys (one workgroup per viewing block adds to them)
     float* dv32;
-    long long acc_b;           // token slots per batch entry (0 for a packed layout: tokens are batch-global)
+    void* dq;
+    void* dk;
+    void* dv;
+    long long dq_b, dq_h, dq_t, dk_b, dk_h, dk_t, dv_b, dv_h, dv_t;
     unsigned q32_b, q32_h, q32_t, k32_b, k32_h, k32_t, v32_b, v32_h, v32_t, o32_b, o32_h, o32_t, g32_b, g32_h, g32_t;
     int B, Nq, Nkv, M, H;
     BrGeom geom;

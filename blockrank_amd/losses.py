@@ -57,6 +57,8 @@ def compute_auxiliary_attention_loss(
     _, N, h1, MH = attention_scores.shape
     assert MH == M * H, "Attention scores last dimension must match M*H"
     rows = bracket_rows(labels, h1)                                  # (B, 2) in [0, h1)
+    if isinstance(attention_scores, LastBlockScores) and attention_scores.needs_grad():
+        attention_scores = attention_scores.dense()          # training: the differentiable logits tensor
     if isinstance(attention_scores, LastBlockScores):
         logits = attention_scores.doc_scores_window(rows, temperature=temperature)
     else:

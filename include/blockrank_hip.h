@@ -208,17 +208,20 @@ int br_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, c
                        const int64_t* out_strides, float scale, void* workspace, size_t workspace_bytes, float* lse,
                        const int64_t* lse_strides, void* stream);
 
-/* Bytes of scratch br_prefill_bwd needs (fp32 accumulators of dq, dk, dv).  token_slots = B*M*H for the padded
- * layout, the packed token count otherwise. */
-size_t br_prefill_bwd_workspace_bytes(int Nq, int Nkv, int D, int64_t token_slots);
+/* Bytes of scratch br_prefill_bwd needs (fp32 dQ sums of the query block's rows, dK and dV sums of the prefix keys, and
+ * rowsum(dO * O) per row and head).  token_slots = B*M*H for the padded layout, the packed token count otherwise. */
+size_t br_prefill_bwd_workspace_bytes(int B, int Nq, int Nkv, int H, int D, int64_t token_slots);
 
 /* Gradients of the attention output with respect to q, k and v (bf16, D 64 or 128):
  *   P = softmax(scale * q.k over visible keys),  dV = P^T dO,  dS = P * (dO V^T - rowsum(dO * O)),
  *   dQ = scale * dS K,  dK = scale * dS^T Q,  dK and dV summed over the query heads of a kv head.
- * q, k, v, out, lse and plan exactly as given to / written by br_prefill_fwd_lse; dout has out's logical shape
- * (B, Nq, S, D) with its own strides; dq (B, Nq, S, D), dk, dv (B, Nkv, S, D) with their strides.  Rows of padded
- * slots receive zeros; dout on padded slots is ignored.  Sums are accumulated in fp32 with atomic adds, so the
- * last bits depend on the order in which workgroups finish. */
+ * q, k, v, out, lse and plan exactly as given to / written by br_prefill_fwd_lse, with lse dense:
+ * lse_strides = (Nq*M*H, M*H) for the padded layout, (0, token_slots) for a packed one.  dout has out's logical
+ * shape (B, Nq, S, D) with its own strides; dq (B, Nq, S, D), dk, dv (B, Nkv, S, D) with their strides.  Rows of
+ * padded slots receive zeros; dout on padded slots is ignored.  Sums with one owner are kept in registers in a
+ * fixed order; dQ of a query block whose key walk is split over several workgroups and dK, dV of the prefix keys
+ * (one workgroup per viewing block) are summed with fp32 atomic adds, so their last bits depend on the order in
+ * which the workgroups finish. */
 int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
                    const int32_t* plan, int B, int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides,
                    const int64_t* k_strides, const int64_t* v_strides, const int64_t* out_strides, const int64_t* dout_strides,

@@ -102,3 +102,67 @@ def test_truncated_ranker_matches_full_forward(kind, dtype):
         assert got.shape == (B, lay.M - 2)
         torch.testing.assert_close(got, want, rtol=2e-3 if dtype == torch.bfloat16 else 1e-4, atol=1e-5)
         assert torch.equal(ranker.rank(ids, valid, pos, labels=lay.labels.to(DEV), k=3), br.rank_documents(want, 3))
+
+
+def test_training_step_gradients_match_eager_autograd():
+    """A training step through the hooks (trainer.py:79-101: language-model loss + auxiliary attention loss on the
+    scoring layer's logits): parameter gradients from the HIP backward against torch autograd through the
+    library's eager attention under the dense mask.  The yardstick is the same step in fp32: the HIP path (bf16)
+    must be about as close to it as the eager path is in bf16 (at most 1.5 times its relative error, and the
+    same direction)."""
+    import copy
+    br.register_blockrank_attention()
+    model = build("mistral", torch.bfloat16)
+    lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
+    lay.labels[:] = -100
+    lay.labels[:, -2:] = 7
+    B, S, M, H = lay.B, lay.S, lay.M, lay.H
+    ids = torch.randint(0, 512, (B, S), generator=torch.Generator().manual_seed(5)).to(DEV)
+    pos = lay.position_ids.to(DEV)
+    valid = lay.valid.to(DEV)
+    labels = lay.labels.to(DEV)
+    answer_ids = torch.tensor([[1], [2]], device=DEV)
+    rows_real = valid.reshape(B, S)
+    probe = torch.randn((B, S, 256), generator=torch.Generator().manual_seed(6)).to(DEV)
+    picked = ("layers.0.self_attn", "layers.1.self_attn.q_proj", "embed_tokens")
+
+    def losses(out, aux_logits):
+        lm = (out.hidden_states[-1].float() * probe)[rows_real].sum() / rows_real.sum()
+        aux = torch.nn.functional.cross_entropy(aux_logits.float(), answer_ids[:, 0])
+        return lm + aux
+
+    def grads(mdl):
+        return {n: p.grad.detach().float().clone() for n, p in mdl.named_parameters() if any(k in n for k in picked)}
+
+    model.set_attn_implementation("default_blockrank")
+    model.zero_grad()
+    out = model(input_ids=ids, position_ids=pos, attention_mask=valid, output_attentions=True, layers_to_return_scores=[1],
+                output_hidden_states=True, use_cache=False)
+    s_last = out.attentions[0]
+    assert isinstance(s_last, torch.Tensor) and s_last.requires_grad, "training returns the differentiable logits tensor"
+    aux_logits = br.compute_auxiliary_attention_loss(s_last, labels, valid, answer_ids=None, return_logits=True)
+    losses(out, aux_logits).backward()
+    ours = grads(model)
+
+    def eager_step(mdl, dtype):
+        ok = torch.as_tensor(orc.allowed(lay.valid.numpy())) | torch.eye(S, dtype=torch.bool)[None]
+        add = torch.zeros(B, 1, S, S, dtype=dtype).masked_fill_(~ok[:, None], torch.finfo(dtype).min).to(DEV)
+        mdl.set_attn_implementation("eager")
+        mdl.zero_grad()
+        ref = mdl(input_ids=ids, position_ids=pos, attention_mask=add, output_attentions=True, output_hidden_states=True, use_cache=False)
+        # the per-document score from the eager probabilities: a softmax restricted to the document columns is the
+        # probabilities renormalised over them (losses.py:56-68)
+        p = ref.attentions[1][:, :, S - 3:S - 1, H:S - H].float()          # rows {bracket - 1, bracket}: the bracket is the first labelled token
+        p = p / p.sum(dim=-1, keepdim=True)
+        logits = p.reshape(B, p.shape[1], 2, M - 2, H).sum(-1).mean(dim=(1, 2)) / 0.05
+        losses(ref, logits).backward()
+        return logits.detach(), grads(mdl)
+
+    logits16, eager16 = eager_step(model, torch.bfloat16)
+    logits32, exact = eager_step(copy.deepcopy(model).float(), torch.float32)
+    assert (aux_logits.float() - logits32).abs().max() <= max(1.5 * (logits16 - logits32).abs().max().item(), 1e-3)
+    for n, w in exact.items():
+        rel = ((ours[n] - w).norm() / w.norm()).item()
+        rel16 = ((eager16[n] - w).norm() / w.norm()).item()
+        cos = torch.nn.functional.cosine_similarity(ours[n].flatten(), w.flatten(), dim=0).item()
+        assert rel <= max(1.5 * rel16, 2e-2) and cos >= 0.99, f"{n}: relative gradient error {rel:.3e} (eager bf16: {rel16:.3e}), cosine {cos:.5f}"

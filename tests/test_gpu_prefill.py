@@ -181,8 +181,13 @@ def test_error_behaviour():
         br.blockrank_attention(q, k, v, torch.ones(1, 2, 8, dtype=torch.bool, device=DEV), 0.1)
     with pytest.raises(NotImplementedError):
         br.blockrank_attention(q.half(), k.half(), v.half(), lay.valid.to(DEV), 0.1)
+    # gradients: bf16 attention has a backward; fp32 inputs and the fused score partials do not
+    # (the reference's kernelised path refuses every backward, blockrank_triton_kernel_attention.py:759-761)
     with pytest.raises(NotImplementedError):
-        br.blockrank_attention(q.clone().requires_grad_(), k, v, lay.valid.to(DEV), 0.1)
+        br.blockrank_attention(q.float().requires_grad_(), k.float(), v.float(), lay.valid.to(DEV), 0.1)
+    with pytest.raises(NotImplementedError):
+        br.blockrank_attention(q.clone().requires_grad_(), k, v, lay.valid.to(DEV), 0.1, score_rows=8)
+    assert br.blockrank_attention(q.clone().requires_grad_(), k, v, lay.valid.to(DEV), 0.1).requires_grad
     with pytest.raises(RuntimeError):
         br.blockrank_attention(q.cpu(), k.cpu(), v.cpu(), br.BlockMask(lay.valid.to(DEV)), 0.1)
     # head dim the kernels do not cover
