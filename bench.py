@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BlockRank attention + per-document score path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5shape|cfg1] [--qk-fp8] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5shape|cfg1] [--qk-fp8] [--backward] [--no-cpu-baseline]
 
 A step is one pass of the hot path over one batch already resident in HBM: the attention hook
 (block-sparse prefill attention of one layer, query/key/value as a Mistral layer hands them over)
@@ -199,6 +199,52 @@ def bench_model(args):
     print(json.dumps(res))
 
 
+def bench_backward(args, br, layout, wl, q, k, v, mask, scale):
+    """Attention training step (bf16): forward + saved log-sum-exp, then dq, dk, dv.  One JSON line; the roofline
+    object prices the backward launches (dQ kernel + dK/dV kernel + their small helpers) at 2.5 times the forward's
+    algorithmic FLOPs: five products per visible pair instead of two."""
+    Nq, D = wl["Nq"], wl["D"]
+    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+    dout = torch.randn((layout.B, layout.S, Nq, D), device=q.device, dtype=q.dtype)
+
+    def step(ev=None):
+        for t in (qq, kk, vv):
+            t.grad = None
+        if ev:
+            ev[0].record()
+        out = br.blockrank_attention(qq, kk, vv, mask, scale)
+        if ev:
+            ev[1].record()
+        out.backward(dout)
+        if ev:
+            ev[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+    pairs_n = layout.unmasked_pairs()
+    flops_bwd = 10.0 * D * pairs_n * Nq
+    tflops = flops_bwd / (bwd_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": f"attention training steps: sequences/sec through forward + backward ({args.workload})",
+        "value": layout.B / (ms_per_step * 1e-3), "unit": "sequences/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": wl["desc"], "name": args.workload, "batch": layout.B, "blocks": layout.M, "block_len": layout.H,
+                   "valid_tokens": layout.valid_tokens, "unmasked_pairs": pairs_n, "pass": "forward + backward"},
+        "forward_us": fwd_ms * 1e3, "backward_us": bwd_ms * 1e3,
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tflops / PEAK_BF16_TFLOPS,
+                     "traffic": None, "kernel": "br_bwd_dq_kernel + br_bwd_dkv_kernel", "flops_per_launch": flops_bwd},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -209,6 +255,8 @@ def main():
     ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
     ap.add_argument("--qk-fp8", action="store_true",
                     help="compute Q K^T in fp8 e4m3 (bf16 workloads with head dim 128; includes the quantisation pass)")
+    ap.add_argument("--backward", action="store_true",
+                    help="time the training step of the attention instead: forward that saves the log-sum-exp, then the backward kernels")
     ap.add_argument("--hf-rope", action="store_true", help="cfg3: keep the model file's own rotary embedding (eight elementwise passes per layer)")
     ap.add_argument("--padded", action="store_true",
                     help="cfg3: feed the reference's padded (B, M, H) batch instead of the packed one")
@@ -251,6 +299,9 @@ def main():
     mask.plan(Nq, Nkv)
     torch.cuda.synchronize()
     plan_ms = (time.perf_counter() - t0) * 1e3
+
+    if args.backward:
+        return bench_backward(args, br, layout, wl, q, k, v, mask, scale)
 
     def step(events=None):
         out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events,
