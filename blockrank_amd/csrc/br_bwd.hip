@@ -246,58 +246,72 @@ struct Bwd {
     }
 
     // ---------------------------------------------------------------------------------------------------------
-    // dK, dV of one 64-key tile of one kv head.  256 threads: wave = (key half kb, head parity hsel).
+    // dK, dV of one 64-key tile of one kv head.  256 threads: wave = (key half kb = wave & 1, side dh = wave >> 1).
+    // The two waves of a key half work on the same step - 32 query rows of one head - and split it: the dh = 0
+    // wave loads the Q rows and computes S = Q K^T, the dh = 1 wave loads the dO rows and computes dP = dO V^T;
+    // they exchange the two 32x32 results through LDS, and then each owns one half of the head dim of dV and dK
+    // (dims [dh D/2, (dh+1) D/2)), whose "lane = dim" operands are transposing reads of the rows the pair has
+    // copied to LDS.  16 MFMAs per wave and step, nothing computed twice; per wave 64 accumulator registers, 32 of
+    // K or V operands, 32 of rows in flight: about 200 in all, so two workgroups share a CU.
     // ---------------------------------------------------------------------------------------------------------
-    static constexpr int dkvLdsBytes = 4 * (2 * rowsBytes + 256);     // per wave: its copy of 32 rows of Q and of dO, their lse and delta
+    static constexpr int xBytes = 2 * 4 * 64 * 16;                        // the pair's two 32x32 fp32 results
+    static constexpr int pairBytes = 2 * rowsBytes + xBytes + 256;        // 32 rows of Q, of dO, the exchange, lse and delta
+    static constexpr int dkvLdsBytes = 2 * pairBytes;
 
     // mq_only < 0: the tile's main workgroup - viewers are the rest of the keys' own block and, for document keys,
     // the query block; mq_only >= 1 (prefix keys only): the rows of block mq_only.  Prefix keys have a workgroup
     // per viewing block, so their sums meet in fp32 buffers (atomic adds); all other keys have one owner, which
     // stores bf16.
     static __device__ __forceinline__ void dkv_tile(const BrBwdParams& p, const BrPlanView& pv, int b, int m, int kt, int kvh, int mq_only, char* smem) {
+        constexpr int NH = ND / 2 > 0 ? ND / 2 : 1;                    // 32-dim blocks a wave owns
+        static_assert(ND % 2 == 0, "the head dim is split in two halves of whole 32-dim blocks");
         const int tid = threadIdx.x;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
-        const int kb = wave & 1, hsel = wave >> 1;
+        const int kb = wave & 1, dh = wave >> 1;
         const int G = p.geom.G, M = p.M;
         const int len_m = pv.len[b * M + m], tok_m = pv.tok[b * M + m];
         const int key0 = kt * BR_BN;
         const int nvalid = len_m - key0 < BR_BN ? len_m - key0 : BR_BN;      // > 0: checked by the caller
-        char* Wq = smem + wave * (2 * rowsBytes + 256);
+        char* Wq = smem + kb * pairBytes;
         char* Wd = Wq + rowsBytes;
-        float* Wl = reinterpret_cast<float*>(Wd + rowsBytes);       // [32] log-sum-exp, [32] delta
+        uint4* X = reinterpret_cast<uint4*>(Wd + rowsBytes);              // [2 sides][4][64 lanes] x 16 bytes
+        float* Wl = reinterpret_cast<float*>(Wd + rowsBytes + xBytes);    // [32] log-sum-exp, [32] delta
 
-        // this wave's 32 keys as operands (lane = key, registers = dims); rows past the real keys are zero
-        bf16x8 kf[NC], vf[NC];
+        // this wave's side: Q rows against K (dh = 0) or dO rows against V (dh = 1)
+        const char* kv_t = reinterpret_cast<const char*>(dh == 0 ? p.k : p.v);
+        const unsigned kv_b = dh == 0 ? p.k32_b : p.v32_b, kv_h = dh == 0 ? p.k32_h : p.v32_h, kv_s = dh == 0 ? p.k32_t : p.v32_t;
+        const char* row_t = reinterpret_cast<const char*>(dh == 0 ? p.q : p.dout);
+        const unsigned row_b = dh == 0 ? p.q32_b : p.g32_b, row_h = dh == 0 ? p.q32_h : p.g32_h, row_s = dh == 0 ? p.q32_t : p.g32_t;
+        const float* stat = dh == 0 ? p.lse : p.delta;
+        char* Wmine = dh == 0 ? Wq : Wd;
+
+        // the wave's 32 keys as operands (lane = key, registers = dims); rows past the real keys are zero
+        bf16x8 ks[NC];
         {
             const int key = kb * 32 + ln;
             const bool on = key < nvalid;
             const unsigned tok = (unsigned)(tok_m + key0 + (on ? key : 0));
-            const char* krow = reinterpret_cast<const char*>(p.k) +
-                               2 * ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh + (unsigned long long)p.k32_t * tok);
-            const char* vrow = reinterpret_cast<const char*>(p.v) +
-                               2 * ((unsigned long long)p.v32_b * (unsigned)b + (unsigned long long)p.v32_h * (unsigned)kvh + (unsigned long long)p.v32_t * tok);
+            const char* row = kv_t + 2 * ((unsigned long long)kv_b * (unsigned)b + (unsigned long long)kv_h * (unsigned)kvh + (unsigned long long)kv_s * tok);
 #pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                kf[c] = as_bf16x8(on ? ld16(krow + c * 32 + lh * 16) : uint4{0u, 0u, 0u, 0u});
-                vf[c] = as_bf16x8(on ? ld16(vrow + c * 32 + lh * 16) : uint4{0u, 0u, 0u, 0u});
-            }
+            for (int c = 0; c < NC; ++c) ks[c] = as_bf16x8(on ? ld16(row + c * 32 + lh * 16) : uint4{0u, 0u, 0u, 0u});
         }
-        f32x16 dk[ND], dv[ND];      // lane = dim 32 db + ln, register v = key kb*32 + 8 (v/4) + 4 lh + v%4
+        f32x16 dk[NH], dv[NH];      // lane = dim 32 (dh NH + j) + ln, register v = key kb*32 + 8 (v/4) + 4 lh + v%4
 #pragma unroll
-        for (int db = 0; db < ND; ++db) dk[db] = dv[db] = zero16();
+        for (int j = 0; j < NH; ++j) dk[j] = dv[j] = zero16();
         const bool half_on = kb * 32 < nvalid;
 
-        // The wave's steps: (32-row block that sees these keys, one of the wave's heads).  Row blocks come from up to
+        // The workgroup's steps: (32-row block that sees these keys, head of the group).  Row blocks come from up to
         // two blocks: the keys' own block from the diagonal on, then the query block (document keys) - or, for a
-        // prefix-key workgroup of a viewing block, that block alone.  Every quantity below is wave-uniform.
+        // prefix-key workgroup of a viewing block, that block alone.  The step sequence is the same for all four
+        // waves (they meet at barriers); whether a key half has something to compute in a step is decided per pair.
         struct Step {
             int r0, nrows, tok, head, self;
         };
         const int blk0 = mq_only < 0 ? m : mq_only;
         const int blk1 = (mq_only < 0 && m > 0 && m < M - 1) ? M - 1 : -1;
-        int seg = (half_on && hsel < G) ? 0 : 2;               // 2 = exhausted
+        int seg = 0;                                                 // 2 = exhausted
         int cur_blk = blk0, cur_len = pv.len[b * M + blk0], cur_tok = pv.tok[b * M + blk0];
-        int rb = mq_only < 0 ? key0 / BR_RB : 0, hl = hsel;
+        int rb = mq_only < 0 ? key0 / BR_RB : 0, hl = 0;
         auto next_step = [&](Step& st) -> bool {
             while (seg < 2) {
                 if (rb * BR_RB >= cur_len) {
@@ -311,161 +325,141 @@ struct Bwd {
                     continue;
                 }
                 const int r0 = rb * BR_RB;
-                const int nrows = cur_len - r0 < BR_RB ? cur_len - r0 : BR_RB;
-                const int self = cur_blk == m;
-                // causal rule on the block's own keys: nothing to do if even the last row precedes this half's first key
-                if (self && r0 + nrows - 1 < key0 + kb * 32) {
-                    ++rb;
-                    continue;
-                }
-                st.r0 = r0; st.nrows = nrows; st.tok = cur_tok + r0; st.head = kvh * G + hl; st.self = self;
-                hl += 2;
-                if (hl >= G) {
-                    hl = hsel;
+                st.r0 = r0;
+                st.nrows = cur_len - r0 < BR_RB ? cur_len - r0 : BR_RB;
+                st.tok = cur_tok + r0;
+                st.head = kvh * G + hl;
+                st.self = cur_blk == m;
+                if (++hl >= G) {
+                    hl = 0;
                     ++rb;
                 }
                 return true;
             }
             return false;
         };
-        // Q and dO rows of a step (lane = row, registers = dims; rows past the block's end repeat its last row and
-        // are masked later), and the rows' log-sum-exp and delta (lane ln holds row ln's)
-        auto load_step = [&](const Step& st, uint4 (&qv)[NC], uint4 (&gv)[NC], float& lse_l, float& delta_l) {
+        // the pair's key half has a pair to compute in this step (causal rule on the block's own keys: nothing if even
+        // the last row precedes the half's first key)
+        auto has_work = [&](const Step& st) { return half_on && !(st.self && st.r0 + st.nrows - 1 < key0 + kb * 32); };
+        // this side's rows of a step (lane = row, registers = dims; rows past the block's end repeat its last row and
+        // are masked later) and the rows' log-sum-exp (dh = 0) or delta (dh = 1); lane ln holds row ln's
+        auto load_step = [&](const Step& st, uint4 (&rv)[NC], float& stat_l) {
             const int r = ln < st.nrows ? ln : st.nrows - 1;
             const unsigned tok = (unsigned)(st.tok + r);
-            const char* qrow = reinterpret_cast<const char*>(p.q) +
-                               2 * ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)st.head + (unsigned long long)p.q32_t * tok);
-            const char* grow = reinterpret_cast<const char*>(p.dout) +
-                               2 * ((unsigned long long)p.g32_b * (unsigned)b + (unsigned long long)p.g32_h * (unsigned)st.head + (unsigned long long)p.g32_t * tok);
+            const char* row = row_t + 2 * ((unsigned long long)row_b * (unsigned)b + (unsigned long long)row_h * (unsigned)st.head + (unsigned long long)row_s * tok);
 #pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                qv[c] = ld16(qrow + c * 32 + lh * 16);
-                gv[c] = ld16(grow + c * 32 + lh * 16);
-            }
-            const long long li = (long long)b * p.lse_b + (long long)st.head * p.lse_h + tok;
-            lse_l = p.lse[li];
-            delta_l = p.delta[li];
+            for (int c = 0; c < NC; ++c) rv[c] = ld16(row + c * 32 + lh * 16);
+            stat_l = stat[(long long)b * p.lse_b + (long long)st.head * p.lse_h + tok];
         };
         {
-            // Per step: copy the rows into the wave's LDS area, S = Q K^T and dP = dO V^T from the registers - after
-            // which the registers are free, so the next step's loads are issued into them and fly while the rest of
-            // this step (softmax terms, dV and dK products, which read the LDS copy) is computed.
+            // Per step: barrier (every wave is done with the previous rows); copy this side's rows to LDS; this side's
+            // product from the registers, result to the exchange - after which the registers are free, so the next
+            // step's loads are issued into them; barrier (rows and both products are in LDS); the other side's
+            // product; softmax terms; dV and dK products of this wave's half of the head dim.
             Step cur, nxt;
-            uint4 qv[NC], gv[NC];
-            float lse_c = 0.f, delta_c = 0.f, lse_n = 0.f, delta_n = 0.f;
+            uint4 rv[NC];
+            float stat_c = 0.f, stat_n = 0.f;
             bool have = next_step(cur);
-            if (have) load_step(cur, qv, gv, lse_c, delta_c);
+            if (have && has_work(cur)) load_step(cur, rv, stat_c);
             while (have) {
                 const bool have_next = next_step(nxt);
-                // (a wave's LDS operations complete in order; the empty asm stops the compiler from reordering them)
-                asm volatile("" ::: "memory");
+                const bool work = has_work(cur);
+                __syncthreads();
+                f32x16 mine = zero16();
+                if (work) {
 #pragma unroll
-                for (int c = 0; c < NC; ++c) {
-                    *reinterpret_cast<uint4*>(Wq + ln * RS + c * 32 + lh * 16) = qv[c];
-                    *reinterpret_cast<uint4*>(Wd + ln * RS + c * 32 + lh * 16) = gv[c];
-                }
-                if (lh == 0) {
-                    Wl[ln] = lse_c;
-                    Wl[32 + ln] = delta_c;
-                }
-                asm volatile("" ::: "memory");
-                f32x16 sn = zero16(), dpn = zero16();
+                    for (int c = 0; c < NC; ++c) *reinterpret_cast<uint4*>(Wmine + ln * RS + c * 32 + lh * 16) = rv[c];
+                    if (lh == 0) Wl[dh * 32 + ln] = stat_c;
 #pragma unroll
-                for (int c = 0; c < NC; ++c) {
-                    sn = mma(as_bf16x8(qv[c]), kf[c], sn);
-                    dpn = mma(as_bf16x8(gv[c]), vf[c], dpn);
-                }
-                if (have_next) load_step(nxt, qv, gv, lse_n, delta_n);
-                // the "lane = dim" operands: all transposing reads are issued here, ahead of the arithmetic that hides
-                // their latency (the compiler keeps each such read next to its use)
-                bf16x8 cd[ND][2], cq[ND][2];
+                    for (int c = 0; c < NC; ++c) mine = mma(as_bf16x8(rv[c]), ks[c], mine);
 #pragma unroll
-                for (int db = 0; db < ND; ++db)
+                    for (int v4 = 0; v4 < 4; ++v4) {
+                        const f32x4 t = {mine[4 * v4], mine[4 * v4 + 1], mine[4 * v4 + 2], mine[4 * v4 + 3]};
+                        *reinterpret_cast<f32x4*>(X + (dh * 4 + v4) * 64 + lane) = t;
+                    }
+                }
+                if (have_next && has_work(nxt)) load_step(nxt, rv, stat_n);
+                __syncthreads();
+                if (work) {
+                    f32x16 other;
+#pragma unroll
+                    for (int v4 = 0; v4 < 4; ++v4) {
+                        const f32x4 t = *reinterpret_cast<const f32x4*>(X + ((1 - dh) * 4 + v4) * 64 + lane);
+                        other[4 * v4] = t[0]; other[4 * v4 + 1] = t[1]; other[4 * v4 + 2] = t[2]; other[4 * v4 + 3] = t[3];
+                    }
+                    const int key = kb * 32 + ln;
+                    const bool key_ok = key < nvalid;
+                    f32x16 pr16, ds16;
+#pragma unroll
+                    for (int v4 = 0; v4 < 4; ++v4) {
+                        // accumulator registers 4 v4 .. 4 v4 + 3 hold rows r0 + 8 v4 + 4 lh + 0..3
+                        const f32x4 l4 = *reinterpret_cast<const f32x4*>(Wl + 8 * v4 + 4 * lh);
+                        const f32x4 d4 = *reinterpret_cast<const f32x4*>(Wl + 32 + 8 * v4 + 4 * lh);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int v = 4 * v4 + e, i = 8 * v4 + 4 * lh + e;
+                            const float s_v = dh == 0 ? mine[v] : other[v], dp_v = dh == 0 ? other[v] : mine[v];
+                            // hidden pairs get exponent -inf, i.e. probability 0, without a branch (every operand is finite)
+                            const bool vis = key_ok && i < cur.nrows && (!cur.self || key0 + key <= cur.r0 + i);
+                            const float pr = __builtin_amdgcn_exp2f(vis ? s_v * p.scale_log2 - l4[e] : -INFINITY);
+                            pr16[v] = pr;
+                            ds16[v] = pr * (dp_v - d4[e]) * p.scale;
+                        }
+                    }
+                    // the "lane = dim" operands of one 16-row step at a time: its reads are issued together, ahead of its products
 #pragma unroll
                     for (int s2 = 0; s2 < 2; ++s2) {
-                        cd[db][s2] = read_col(Wd, 16 * s2, db, lane);
-                        cq[db][s2] = read_col(Wq, 16 * s2, db, lane);
+                        const bf16x8 pa = pack8(pr16, s2), da = pack8(ds16, s2);
+                        bf16x8 cd[NH], cq[NH];
+#pragma unroll
+                        for (int j = 0; j < NH; ++j) {
+                            cd[j] = read_col(Wd, 16 * s2, dh * NH + j, lane);
+                            cq[j] = read_col(Wq, 16 * s2, dh * NH + j, lane);
+                        }
+#pragma unroll
+                        for (int j = 0; j < NH; ++j) {
+                            dv[j] = mma(pa, cd[j], dv[j]);
+                            dk[j] = mma(da, cq[j], dk[j]);
+                        }
                     }
-                const int key = kb * 32 + ln;
-                const bool key_ok = key < nvalid;
-#pragma unroll
-                for (int v4 = 0; v4 < 4; ++v4) {
-                    // accumulator registers 4 v4 .. 4 v4 + 3 hold rows r0 + 8 v4 + 4 lh + 0..3
-                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(Wl + 8 * v4 + 4 * lh);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(Wl + 32 + 8 * v4 + 4 * lh);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int v = 4 * v4 + e, i = 8 * v4 + 4 * lh + e;
-                        // hidden pairs get exponent -inf, i.e. probability 0, without a branch (every operand is finite)
-                        const bool vis = key_ok && i < cur.nrows && (!cur.self || key0 + key <= cur.r0 + i);
-                        const float pr = __builtin_amdgcn_exp2f(vis ? sn[v] * p.scale_log2 - l4[e] : -INFINITY);
-                        sn[v] = pr;
-                        dpn[v] = pr * (dpn[v] - d4[e]) * p.scale;
-                    }
-                }
-                const bf16x8 p0 = pack8(sn, 0), p1 = pack8(sn, 1), d0 = pack8(dpn, 0), d1 = pack8(dpn, 1);
-#pragma unroll
-                for (int db = 0; db < ND; ++db) {
-                    dv[db] = mma(p0, cd[db][0], dv[db]);
-                    dk[db] = mma(d0, cq[db][0], dk[db]);
-                }
-#pragma unroll
-                for (int db = 0; db < ND; ++db) {
-                    dv[db] = mma(p1, cd[db][1], dv[db]);
-                    dk[db] = mma(d1, cq[db][1], dk[db]);
                 }
                 cur = nxt;
-                lse_c = lse_n;
-                delta_c = delta_n;
+                stat_c = stat_n;
                 have = have_next;
             }
         }
 
+        if (!half_on) return;
         if (m == 0 && M > 1) {
             // prefix keys: add into the fp32 buffers [b][kv head][key][D]
-            float* k32 = p.dk32 + (((long long)b * p.Nkv + kvh) * p.H + key0 + kb * 32 + 4 * lh) * D + ln;
-            float* v32 = p.dv32 + (((long long)b * p.Nkv + kvh) * p.H + key0 + kb * 32 + 4 * lh) * D + ln;
-            if (half_on) {
+            const long long base = (((long long)b * p.Nkv + kvh) * p.H + key0 + kb * 32 + 4 * lh) * D + dh * NH * 32 + ln;
 #pragma unroll
-                for (int db = 0; db < ND; ++db)
+            for (int j = 0; j < NH; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int kr = 8 * (v >> 2) + (v & 3);
-                        if (kb * 32 + 4 * lh + kr < nvalid) {
-                            unsafeAtomicAdd(k32 + kr * D + db * 32, dk[db][v]);
-                            unsafeAtomicAdd(v32 + kr * D + db * 32, dv[db][v]);
-                        }
+                for (int v = 0; v < 16; ++v) {
+                    const int kr = 8 * (v >> 2) + (v & 3);
+                    if (kb * 32 + 4 * lh + kr < nvalid) {
+                        unsafeAtomicAdd(p.dk32 + base + kr * D + j * 32, dk[j][v]);
+                        unsafeAtomicAdd(p.dv32 + base + kr * D + j * 32, dv[j][v]);
                     }
-            }
+                }
             return;
         }
-        // sum the two head parities of each key half through LDS (dK, then dV), then store bf16
-        float* red = reinterpret_cast<float*>(smem);               // [2 halves][32 keys][D] fp32 = 2 * 32 * D * 4 bytes
-        static_assert(2 * 32 * D * 4 <= dkvLdsBytes, "reduction buffer must fit the waves' row copies");
-        auto reduce_store = [&](f32x16 (&acc)[ND], void* out, long long s_b, long long s_h, long long s_t) {
-            __syncthreads();
-            if (hsel == 1) {
+        // every other key has this one owner: store bf16
+        __bf16* dkp = reinterpret_cast<__bf16*>(p.dk) + (long long)b * p.dk_b + (long long)kvh * p.dk_h +
+                      (long long)(tok_m + key0 + kb * 32 + 4 * lh) * p.dk_t + dh * NH * 32 + ln;
+        __bf16* dvp = reinterpret_cast<__bf16*>(p.dv) + (long long)b * p.dv_b + (long long)kvh * p.dv_h +
+                      (long long)(tok_m + key0 + kb * 32 + 4 * lh) * p.dv_t + dh * NH * 32 + ln;
 #pragma unroll
-                for (int db = 0; db < ND; ++db)
+        for (int j = 0; j < NH; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) red[(kb * 32 + 8 * (v >> 2) + 4 * lh + (v & 3)) * D + db * 32 + ln] = acc[db][v];
+            for (int v = 0; v < 16; ++v) {
+                const int kr = 8 * (v >> 2) + (v & 3);
+                if (kb * 32 + 4 * lh + kr < nvalid) {
+                    dkp[(long long)kr * p.dk_t + j * 32] = (__bf16)dk[j][v];
+                    dvp[(long long)kr * p.dv_t + j * 32] = (__bf16)dv[j][v];
+                }
             }
-            __syncthreads();
-            if (hsel == 0) {
-                __bf16* dst = reinterpret_cast<__bf16*>(out) + (long long)b * s_b + (long long)kvh * s_h +
-                              (long long)(tok_m + key0 + kb * 32 + 4 * lh) * s_t + ln;
-#pragma unroll
-                for (int db = 0; db < ND; ++db)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int kr = 8 * (v >> 2) + (v & 3);
-                        const float x = acc[db][v] + red[(kb * 32 + 4 * lh + kr) * D + db * 32 + ln];
-                        if (kb * 32 + 4 * lh + kr < nvalid) dst[(long long)kr * s_t + db * 32] = (__bf16)x;
-                    }
-            }
-        };
-        reduce_store(dk, p.dk, p.dk_b, p.dk_h, p.dk_t);
-        reduce_store(dv, p.dv, p.dv_b, p.dv_h, p.dv_t);
     }
 };
 
@@ -483,7 +477,7 @@ __global__ __launch_bounds__(MAXW * 64, MAXW <= 4 ? 2 : 1) void br_bwd_dq_kernel
 // blockIdx.x enumerates (unit, sequence b, kv head, key tile): units 0 .. M-1 are the blocks' main workgroups, units
 // M .. 2M-2 the workgroups that take the rows of blocks 1 .. M-1 to the prefix keys.
 template <int D>
-__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void br_bwd_dkv_kernel(BrBwdParams p) {
+__global__ __launch_bounds__(256, 2) void br_bwd_dkv_kernel(BrBwdParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     const int KT = (p.H + BR_BN - 1) / BR_BN;
