@@ -148,37 +148,71 @@ struct Bwd {
         const bool table = it.pe > 1;
         const int nprev = it.nprev;
         const int f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
-        for (int f = it.f_lo; f < f_end; ++f) {
-            const bool self = f >= nprev;
-            int tok0, nvalid, key0 = 0;
-            if (!self) {
-                if (table) {
-                    const int2 d = tiles_b[f];
-                    tok0 = d.x;
-                    nvalid = d.y;
+        // The walk is software-pipelined: a thread's pieces of the next tile are loaded into registers while the
+        // current tile (in LDS) is computed.
+        struct Tile {
+            int tok0, nvalid, key0, self;
+        };
+        int f = it.f_lo;
+        auto next_tile = [&](Tile& t) -> bool {
+            while (f < f_end) {
+                const int fi = f++;
+                t.self = fi >= nprev;
+                t.key0 = 0;
+                if (!t.self) {
+                    if (table) {
+                        const int2 d = tiles_b[fi];
+                        t.tok0 = d.x;
+                        t.nvalid = d.y;
+                    } else {
+                        t.tok0 = it.tok0 + fi * BR_BN;
+                        t.nvalid = it.len0 - fi * BR_BN < BR_BN ? it.len0 - fi * BR_BN : BR_BN;
+                    }
                 } else {
-                    tok0 = it.tok0 + f * BR_BN;
-                    nvalid = it.len0 - f * BR_BN < BR_BN ? it.len0 - f * BR_BN : BR_BN;
+                    t.key0 = (fi - nprev) * BR_BN;
+                    if (t.key0 >= self_end) {
+                        f = f_end;
+                        return false;
+                    }
+                    t.tok0 = it.tok_m + t.key0;
+                    t.nvalid = self_end - t.key0 < BR_BN ? self_end - t.key0 : BR_BN;
                 }
-            } else {
-                key0 = (f - nprev) * BR_BN;
-                if (key0 >= self_end) break;
-                tok0 = it.tok_m + key0;
-                nvalid = self_end - key0 < BR_BN ? self_end - key0 : BR_BN;
+                if (t.nvalid > 0) return true;
             }
-            if (nvalid <= 0) continue;
-            // stage the tile: rows past its real keys are zero
-            __syncthreads();                       // every wave has finished with the previous tile
-            for (int idx = tid; idx < BR_BN * CPR; idx += NT) {
+            return false;
+        };
+        constexpr int NPC = BR_BN * CPR / 256;     // 16-byte pieces of K (and of V) per thread and tile (at least 256 threads)
+        uint4 kreg[NPC], vreg[NPC];
+        auto load_tile = [&](const Tile& t) {      // rows past the tile's real keys are zero
+#pragma unroll
+            for (int i = 0; i < NPC; ++i) {
+                const int idx = tid + i * NT;
                 const int r = idx / CPR, c = idx - r * CPR;
-                uint4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-                if (r < nvalid) {
-                    kk = ld16(kbase + 2 * ((long long)(tok0 + r) * p.k32_t + c * 8));
-                    vv = ld16(vbase + 2 * ((long long)(tok0 + r) * p.v32_t + c * 8));
+                kreg[i] = vreg[i] = uint4{0u, 0u, 0u, 0u};
+                if (idx < BR_BN * CPR && r < t.nvalid) {
+                    kreg[i] = ld16(kbase + 2 * ((long long)(t.tok0 + r) * p.k32_t + c * 8));
+                    vreg[i] = ld16(vbase + 2 * ((long long)(t.tok0 + r) * p.v32_t + c * 8));
                 }
-                *reinterpret_cast<uint4*>(Ks + r * RS + c * 16) = kk;
-                *reinterpret_cast<uint4*>(Vs + r * RS + c * 16) = vv;
             }
+        };
+        Tile cur, nxt;
+        bool have = next_tile(cur);
+        if (have) load_tile(cur);
+        while (have) {
+            const bool self = cur.self;
+            const int nvalid = cur.nvalid, key0 = cur.key0;
+            __syncthreads();                       // every wave has finished with the previous tile
+#pragma unroll
+            for (int i = 0; i < NPC; ++i) {
+                const int idx = tid + i * NT;
+                const int r = idx / CPR, c = idx - r * CPR;
+                if (idx < BR_BN * CPR) {
+                    *reinterpret_cast<uint4*>(Ks + r * RS + c * 16) = kreg[i];
+                    *reinterpret_cast<uint4*>(Vs + r * RS + c * 16) = vreg[i];
+                }
+            }
+            const bool have_next = next_tile(nxt);
+            if (have_next) load_tile(nxt);
             __syncthreads();
 
             // 32-key halves this wave needs: limited by the real keys and, on the block's own keys, by the diagonal
@@ -196,12 +230,6 @@ struct Bwd {
                     st = mma(read_row(Ks, kb * 32, c, ln, lh), qf[c], st);
                     dpt = mma(read_row(Vs, kb * 32, c, ln, lh), dof[c], dpt);
                 }
-                // K as "lane = dim" operand: the transposing reads are issued ahead of the arithmetic that hides them
-                bf16x8 kc[2][ND];
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-#pragma unroll
-                    for (int db = 0; db < ND; ++db) kc[s][db] = read_col(Ks, kb * 32 + 16 * s, db, lane);
                 const int lim_c = self ? row0 + ln - key0 + 1 : BR_BN;                 // keys [0, lim) of the tile are visible
                 int lim = nvalid < lim_c ? nvalid : lim_c;
                 if (row0 + ln >= len_m) lim = 0;
@@ -215,10 +243,16 @@ struct Bwd {
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     const bf16x8 a = pack8(st, s);
+                    // K as "lane = dim" operand of this 16-key step: the transposing reads are issued together, ahead of the products
+                    bf16x8 kc[ND];
 #pragma unroll
-                    for (int db = 0; db < ND; ++db) dq[db] = mma(a, kc[s][db], dq[db]);
+                    for (int db = 0; db < ND; ++db) kc[db] = read_col(Ks, kb * 32 + 16 * s, db, lane);
+#pragma unroll
+                    for (int db = 0; db < ND; ++db) dq[db] = mma(a, kc[db], dq[db]);
                 }
             }
+            cur = nxt;
+            have = have_next;
         }
         // dQ of this wave's rows: lane = dim 32 db + ln, register v = row 8 (v/4) + 4 lh + v%4
         if (!rb_active) return;
