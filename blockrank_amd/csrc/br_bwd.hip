@@ -391,13 +391,14 @@ struct Bwd {
             // step's loads are issued into them; barrier (rows and both products are in LDS); the other side's
             // product; softmax terms; dV and dK products of this wave's half of the head dim.
             Step cur, nxt;
-            uint4 rv[NC];
+            uint4 rv[NC], rn[NC];
             float stat_c = 0.f, stat_n = 0.f;
             bool have = next_step(cur);
             if (have && has_work(cur)) load_step(cur, rv, stat_c);
             while (have) {
                 const bool have_next = next_step(nxt);
                 const bool work = has_work(cur);
+                if (have_next && has_work(nxt)) load_step(nxt, rn, stat_n);
                 __syncthreads();
                 f32x16 mine = zero16();
                 if (work) {
@@ -412,7 +413,6 @@ struct Bwd {
                         *reinterpret_cast<f32x4*>(X + (dh * 4 + v4) * 64 + lane) = t;
                     }
                 }
-                if (have_next && has_work(nxt)) load_step(nxt, rv, stat_n);
                 __syncthreads();
                 if (work) {
                     f32x16 other;
@@ -459,6 +459,8 @@ struct Bwd {
                 }
                 cur = nxt;
                 stat_c = stat_n;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) rv[c] = rn[c];
                 have = have_next;
             }
         }
