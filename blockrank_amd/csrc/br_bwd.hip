@@ -41,6 +41,9 @@ __device__ inline bf16x8 as_bf16x8(uint4 u) {
     c.u = u;
     return c.v;
 }
+// Workgroup barrier that waits for this wave's LDS operations only.  __syncthreads() also waits for its outstanding
+// global loads, which would make every barrier wait for the rows requested ahead for the next step.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __device__ inline f32x16 mma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 __device__ inline f32x16 zero16() {
     f32x16 z;
@@ -201,7 +204,7 @@ struct Bwd {
         while (have) {
             const bool self = cur.self;
             const int nvalid = cur.nvalid, key0 = cur.key0;
-            __syncthreads();                       // every wave has finished with the previous tile
+            lds_barrier();                         // every wave has finished with the previous tile
 #pragma unroll
             for (int i = 0; i < NPC; ++i) {
                 const int idx = tid + i * NT;
@@ -213,7 +216,7 @@ struct Bwd {
             }
             const bool have_next = next_tile(nxt);
             if (have_next) load_tile(nxt);
-            __syncthreads();
+            lds_barrier();
 
             // 32-key halves this wave needs: limited by the real keys and, on the block's own keys, by the diagonal
             int nkb = (nvalid + 31) >> 5;
@@ -399,7 +402,7 @@ struct Bwd {
                 const bool have_next = next_step(nxt);
                 const bool work = has_work(cur);
                 if (have_next && has_work(nxt)) load_step(nxt, rn, stat_n);
-                __syncthreads();
+                lds_barrier();
                 f32x16 mine = zero16();
                 if (work) {
 #pragma unroll
@@ -413,7 +416,7 @@ struct Bwd {
                         *reinterpret_cast<f32x4*>(X + (dh * 4 + v4) * 64 + lane) = t;
                     }
                 }
-                __syncthreads();
+                lds_barrier();
                 if (work) {
                     f32x16 other;
 #pragma unroll
@@ -422,24 +425,33 @@ struct Bwd {
                         other[4 * v4] = t[0]; other[4 * v4 + 1] = t[1]; other[4 * v4 + 2] = t[2]; other[4 * v4 + 3] = t[3];
                     }
                     const int key = kb * 32 + ln;
-                    const bool key_ok = key < nvalid;
                     f32x16 pr16, ds16;
+                    // most steps see every pair (whole key half, whole row block, nothing above the diagonal): they
+                    // skip the per-pair visibility test.  sa / da are S and dP whichever side computed them.
+                    const bool all_visible = nvalid - kb * 32 >= 32 && cur.nrows == BR_RB && (!cur.self || key0 + kb * 32 + 31 <= cur.r0);
+                    auto terms = [&](const f32x16& sa, const f32x16& da) {
 #pragma unroll
-                    for (int v4 = 0; v4 < 4; ++v4) {
-                        // accumulator registers 4 v4 .. 4 v4 + 3 hold rows r0 + 8 v4 + 4 lh + 0..3
-                        const f32x4 l4 = *reinterpret_cast<const f32x4*>(Wl + 8 * v4 + 4 * lh);
-                        const f32x4 d4 = *reinterpret_cast<const f32x4*>(Wl + 32 + 8 * v4 + 4 * lh);
+                        for (int v4 = 0; v4 < 4; ++v4) {
+                            // accumulator registers 4 v4 .. 4 v4 + 3 hold rows r0 + 8 v4 + 4 lh + 0..3
+                            const f32x4 l4 = *reinterpret_cast<const f32x4*>(Wl + 8 * v4 + 4 * lh);
+                            const f32x4 d4 = *reinterpret_cast<const f32x4*>(Wl + 32 + 8 * v4 + 4 * lh);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int v = 4 * v4 + e, i = 8 * v4 + 4 * lh + e;
-                            const float s_v = dh == 0 ? mine[v] : other[v], dp_v = dh == 0 ? other[v] : mine[v];
-                            // hidden pairs get exponent -inf, i.e. probability 0, without a branch (every operand is finite)
-                            const bool vis = key_ok && i < cur.nrows && (!cur.self || key0 + key <= cur.r0 + i);
-                            const float pr = __builtin_amdgcn_exp2f(vis ? s_v * p.scale_log2 - l4[e] : -INFINITY);
-                            pr16[v] = pr;
-                            ds16[v] = pr * (dp_v - d4[e]) * p.scale;
+                            for (int e = 0; e < 4; ++e) {
+                                const int v = 4 * v4 + e, i = 8 * v4 + 4 * lh + e;
+                                float x = sa[v] * p.scale_log2 - l4[e];
+                                if (!all_visible) {
+                                    // hidden pairs get exponent -inf, i.e. probability 0, without a branch (every operand is finite)
+                                    const bool vis = key < nvalid && i < cur.nrows && (!cur.self || key0 + key <= cur.r0 + i);
+                                    x = vis ? x : -INFINITY;
+                                }
+                                const float pr = __builtin_amdgcn_exp2f(x);
+                                pr16[v] = pr;
+                                ds16[v] = pr * (da[v] - d4[e]) * p.scale;
+                            }
                         }
-                    }
+                    };
+                    if (dh == 0) terms(mine, other);
+                    else terms(other, mine);
                     // the "lane = dim" operands of one 16-row step at a time: its reads are issued together, ahead of its products
 #pragma unroll
                     for (int s2 = 0; s2 < 2; ++s2) {
