@@ -98,3 +98,17 @@ def test_long_document_list_splits_the_query_walk():
 
 def test_packed_layout():
     _check(synthetic.make_layout([[40, 100, 160, 33, 192, 20], [64, 7, 150, 90, 0, 31]]), 8, 2, 128, seed=16, packed=True)
+
+
+def test_random_layouts():
+    """Seeded random block layouts (empty, one-token, tile-edge and long blocks; every head grouping; both head
+    dims), the same generator as the forward's randomised test."""
+    from tests.test_gpu_random_layouts import _cases
+    for it, lens, G, Nkv, D in _cases(seed=23, n=16):
+        lay = synthetic.make_layout(lens)
+        if lay.S > 2600:                                   # keep the dense float64 oracle within seconds
+            continue
+        try:
+            _check(lay, G * Nkv, Nkv, D, seed=100 + it)
+        except AssertionError as e:
+            raise AssertionError(f"case {it}: lengths {lens}, {G} heads per kv head, {Nkv} kv heads, D={D}: {e}") from e
