@@ -283,33 +283,33 @@ struct Bwd {
     }
 
     // ---------------------------------------------------------------------------------------------------------
-    // dK, dV of one 64-key tile of one kv head.  256 threads: wave = (key half kb = wave & 1, side dh = wave >> 1).
-    // The two waves of a key half work on the same step - 32 query rows of one head - and split it: the dh = 0
+    // dK, dV of one 32-key half (kb) of a 64-key tile of one kv head.  128 threads: wave = side dh.
+    // The two waves work on the same step - 32 query rows of one head - and split it: the dh = 0
     // wave loads the Q rows and computes S = Q K^T, the dh = 1 wave loads the dO rows and computes dP = dO V^T;
     // they exchange the two 32x32 results through LDS, and then each owns one half of the head dim of dV and dK
     // (dims [dh D/2, (dh+1) D/2)), whose "lane = dim" operands are transposing reads of the rows the pair has
     // copied to LDS.  16 MFMAs per wave and step, nothing computed twice; per wave 64 accumulator registers, 32 of
-    // K or V operands, 32 of rows in flight: about 200 in all, so two workgroups share a CU.
+    // K or V operands, 32 of rows in flight: about 200 in all, so four workgroups share a CU.
     // ---------------------------------------------------------------------------------------------------------
     static constexpr int xBytes = 2 * 4 * 64 * 16;                        // the pair's two 32x32 fp32 results
     static constexpr int pairBytes = 2 * rowsBytes + xBytes + 256;        // 32 rows of Q, of dO, the exchange, lse and delta
-    static constexpr int dkvLdsBytes = 2 * pairBytes;
+    static constexpr int dkvLdsBytes = pairBytes;
 
     // mq_only < 0: the tile's main workgroup - viewers are the rest of the keys' own block and, for document keys,
     // the query block; mq_only >= 1 (prefix keys only): the rows of block mq_only.  Prefix keys have a workgroup
     // per viewing block, so their sums meet in fp32 buffers (atomic adds); all other keys have one owner, which
     // stores bf16.
-    static __device__ __forceinline__ void dkv_tile(const BrBwdParams& p, const BrPlanView& pv, int b, int m, int kt, int kvh, int mq_only, char* smem) {
+    static __device__ __forceinline__ void dkv_tile(const BrBwdParams& p, const BrPlanView& pv, int b, int m, int kt, int kb, int kvh, int mq_only, char* smem) {
         constexpr int NH = ND / 2 > 0 ? ND / 2 : 1;                    // 32-dim blocks a wave owns
         static_assert(ND % 2 == 0, "the head dim is split in two halves of whole 32-dim blocks");
         const int tid = threadIdx.x;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, ln = lane & 31, lh = lane >> 5;
-        const int kb = wave & 1, dh = wave >> 1;
+        const int dh = wave;
         const int G = p.geom.G, M = p.M;
         const int len_m = pv.len[b * M + m], tok_m = pv.tok[b * M + m];
         const int key0 = kt * BR_BN;
-        const int nvalid = len_m - key0 < BR_BN ? len_m - key0 : BR_BN;      // > 0: checked by the caller
-        char* Wq = smem + kb * pairBytes;
+        const int nvalid = len_m - key0 < BR_BN ? len_m - key0 : BR_BN;      // > kb * 32: checked by the caller
+        char* Wq = smem;
         char* Wd = Wq + rowsBytes;
         uint4* X = reinterpret_cast<uint4*>(Wd + rowsBytes);              // [2 sides][4][64 lanes] x 16 bytes
         float* Wl = reinterpret_cast<float*>(Wd + rowsBytes + xBytes);    // [32] log-sum-exp, [32] delta
@@ -339,8 +339,8 @@ struct Bwd {
 
         // The workgroup's steps: (32-row block that sees these keys, head of the group).  Row blocks come from up to
         // two blocks: the keys' own block from the diagonal on, then the query block (document keys) - or, for a
-        // prefix-key workgroup of a viewing block, that block alone.  The step sequence is the same for all four
-        // waves (they meet at barriers); whether a key half has something to compute in a step is decided per pair.
+        // prefix-key workgroup of a viewing block, that block alone.  The step sequence is the same for both waves
+        // (they meet at barriers).
         struct Step {
             int r0, nrows, tok, head, self;
         };
@@ -522,14 +522,16 @@ __global__ __launch_bounds__(MAXW * 64, MAXW <= 4 ? 2 : 1) void br_bwd_dq_kernel
     Bwd<D>::dq_item(p, pv, it, hg, smem, blockDim.x >> 6);
 }
 
-// blockIdx.x enumerates (unit, sequence b, kv head, key tile): units 0 .. M-1 are the blocks' main workgroups, units
-// M .. 2M-2 the workgroups that take the rows of blocks 1 .. M-1 to the prefix keys.
+// blockIdx.x enumerates (unit, sequence b, kv head, key tile, 32-key half): units 0 .. M-1 are the blocks' main
+// workgroups, units M .. 2M-2 the workgroups that take the rows of blocks 1 .. M-1 to the prefix keys.
 template <int D>
-__global__ __launch_bounds__(256, 2) void br_bwd_dkv_kernel(BrBwdParams p) {
+__global__ __launch_bounds__(128, 2) void br_bwd_dkv_kernel(BrBwdParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     const int KT = (p.H + BR_BN - 1) / BR_BN;
     int idx = blockIdx.x;
+    const int kb = idx & 1;
+    idx >>= 1;
     const int kt = idx % KT;
     idx /= KT;
     const int kvh = idx % p.Nkv;
@@ -538,7 +540,7 @@ __global__ __launch_bounds__(256, 2) void br_bwd_dkv_kernel(BrBwdParams p) {
     const int m = unit < p.M ? unit : 0, mq_only = unit < p.M ? -1 : unit - p.M + 1;
     const int len_m = pv.len[b * p.M + m];
     // padded slots of this block (dk and dv of this kv head): zeros, written by the block's first workgroup
-    if (kt == 0 && mq_only < 0 && !pv.hdr[BR_PH_PACKED]) {
+    if (kt == 0 && kb == 0 && mq_only < 0 && !pv.hdr[BR_PH_PACKED]) {
         const int st = pv.start[b * p.M + m], npad = p.H - len_m;
         constexpr int CP8 = D / 8;
         const uint4 z = {0u, 0u, 0u, 0u};
@@ -551,8 +553,8 @@ __global__ __launch_bounds__(256, 2) void br_bwd_dkv_kernel(BrBwdParams p) {
             *reinterpret_cast<uint4*>(vb_ + pos * p.dv_t + c8 * 8) = z;
         }
     }
-    if (kt * BR_BN >= len_m) return;
-    Bwd<D>::dkv_tile(p, pv, b, m, kt, kvh, mq_only, smem);
+    if (kt * BR_BN + kb * 32 >= len_m) return;           // no real key in this half
+    Bwd<D>::dkv_tile(p, pv, b, m, kt, kb, kvh, mq_only, smem);
 }
 
 __global__ __launch_bounds__(256) void br_fill_zero_kernel(uint4* p, size_t n16) {
@@ -644,7 +646,7 @@ int launch_all(const BrBwdParams& p, int NW, int n_cu, hipStream_t stream) {
         armed = true;
     }
     const int KT = (p.H + BR_BN - 1) / BR_BN;
-    hipLaunchKernelGGL((br_bwd_dkv_kernel<D>), dim3((2 * p.M - 1) * p.B * p.Nkv * KT), dim3(256), lds, stream, p);
+    hipLaunchKernelGGL((br_bwd_dkv_kernel<D>), dim3((2 * p.M - 1) * p.B * p.Nkv * KT * 2), dim3(128), lds, stream, p);
     hipLaunchKernelGGL((br_bwd_dq_finish_kernel<D>), dim3(n_cu * 4), dim3(256), 0, stream, p);
     return 0;
 }
