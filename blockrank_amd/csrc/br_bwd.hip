@@ -512,7 +512,7 @@ struct Bwd {
 };
 
 template <int D, int MAXW>
-__global__ __launch_bounds__(MAXW * 64, MAXW <= 4 ? 2 : 1) void br_bwd_dq_kernel(BrBwdParams p) {
+__global__ __launch_bounds__(MAXW * 64, MAXW <= 4 ? (D == 64 ? 3 : 2) : 1) void br_bwd_dq_kernel(BrBwdParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const BrGeom& ge = p.geom;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(MAXW * 64, MAXW <= 4 ? 2 : 1) void br_bwd_dq_kernel
 // blockIdx.x enumerates (unit, sequence b, kv head, key tile, 32-key half): units 0 .. M-1 are the blocks' main
 // workgroups, units M .. 2M-2 the workgroups that take the rows of blocks 1 .. M-1 to the prefix keys.
 template <int D>
-__global__ __launch_bounds__(128, 2) void br_bwd_dkv_kernel(BrBwdParams p) {
+__global__ __launch_bounds__(128, D == 64 ? 3 : 2) void br_bwd_dkv_kernel(BrBwdParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     const int KT = (p.H + BR_BN - 1) / BR_BN;
