@@ -105,6 +105,37 @@ def cpu_baseline(layout, q, k, v, scale, dtype, budget_s=12.0):
                 ms_per_request=med * 1e3)
 
 
+def cpu_baseline_backward(layout, q, k, v, dout, scale, dtype, budget_s=12.0):
+    """The same for the training step: forward of the oracle's restatement of the reference's three-call SDPA
+    algorithm plus torch autograd through it (how the reference's trainable hooks are differentiated), on the
+    host cores, for the first sequence of the batch."""
+    from oracle import blockrank_oracle as orc
+    import numpy as np
+    torch.set_num_threads(os.cpu_count() if "OMP_NUM_THREADS" not in os.environ else int(os.environ["OMP_NUM_THREADS"]))
+    q1, k1, v1 = (t[:1].detach().to("cpu", dtype).contiguous().requires_grad_(True) for t in (q, k, v))
+    g1 = dout[:1].detach().to("cpu", dtype).contiguous()
+    m5 = orc.additive_mask(layout.valid[:1], dtype)
+
+    def one():
+        for t in (q1, k1, v1):
+            t.grad = None
+        out, _ = orc.sdpa_blockrank_forward(q1, k1, v1, m5, scale)
+        out.backward(g1)
+
+    one()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return dict(value=1.0 / med, unit="sequences/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"first sequence of the batch ({int(layout.lengths[0].sum())} tokens), {str(dtype).replace('torch.', '')}, forward + "
+                       f"autograd backward, median of {len(times)} runs, {med * 1e3:.1f} ms per sequence",
+                ms_per_sequence=med * 1e3)
+
+
 def bench_model(args):
     """cfg3: the truncated ranking forward of a Mistral-7B-shaped model with random weights."""
     import blockrank_amd as br
@@ -233,7 +264,7 @@ def bench_backward(args, br, layout, wl, q, k, v, mask, scale):
     pairs_n = layout.unmasked_pairs()
     flops_bwd = 10.0 * D * pairs_n * Nq
     tflops = flops_bwd / (bwd_ms * 1e-3) / 1e12
-    print(json.dumps({
+    res = {
         "metric": f"attention training steps: sequences/sec through forward + backward ({args.workload})",
         "value": layout.B / (ms_per_step * 1e-3), "unit": "sequences/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -242,7 +273,11 @@ def bench_backward(args, br, layout, wl, q, k, v, mask, scale):
         "forward_us": fwd_ms * 1e3, "backward_us": bwd_ms * 1e3,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tflops / PEAK_BF16_TFLOPS,
                      "traffic": None, "kernel": "br_bwd_dq_kernel + br_bwd_dkv_kernel", "flops_per_launch": flops_bwd},
-    }))
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline_backward(layout, q, k, v, dout, scale, q.dtype)
+        res["cpu_baseline"]["gpu_over_cpu"] = res["value"] / res["cpu_baseline"]["value"]
+    print(json.dumps(res))
 
 
 def main():
