@@ -249,6 +249,7 @@ class _AttentionWithGrad(torch.autograd.Function):
         return out
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, dout):
         q, k, v, out, lse = ctx.saved_tensors
         bm = ctx.bm
@@ -564,6 +565,7 @@ class _LastLogitsWithGrad(torch.autograd.Function):
         return last_block_logits(query.detach(), key.detach(), bm, rows, scaling, neg=neg)
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, ds):
         query, key, rows = ctx.saved_tensors
         bm = ctx.bm
