@@ -335,6 +335,14 @@ def main():
     torch.cuda.synchronize()
     plan_ms = (time.perf_counter() - t0) * 1e3
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     if args.backward:
         return bench_backward(args, br, layout, wl, q, k, v, mask, scale)
 
@@ -343,14 +351,6 @@ def main():
                                                       qk_fp8=args.qk_fp8)
         scores = handle.doc_scores_window(rows16, temperature=0.05) if handle is not None else None
         return out, scores
-
-    if args.calibrate_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
 
     for _ in range(args.warmup):
         step()

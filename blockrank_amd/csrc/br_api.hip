@@ -389,7 +389,6 @@ int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out,
     BrGeom g;
     int nw;
     make_geom(Nq, Nkv, &g, &nw);
-    if ((long long)M * B * Nkv * ((H + BR_BN - 1) / BR_BN) >= (1LL << 31)) return fail(BR_ERR_ARG, "batch too large for one backward launch");
     BrBwdParams p;
     p.q = q; p.k = k; p.v = v; p.out = out; p.dout = dout; p.plan = plan; p.lse = lse;
     p.lse_b = lse_strides[0]; p.lse_h = lse_strides[1];
@@ -397,7 +396,7 @@ int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out,
     p.dk32 = p.dq32 + (size_t)B * Nq * H * D;
     p.dv32 = p.dk32 + (size_t)B * Nkv * H * D;
     p.delta = reinterpret_cast<float*>(static_cast<char*>(workspace) + up256((size_t)B * (Nq + 2 * Nkv) * H * D * sizeof(float)));
-    if ((long long)(2 * M - 1) * B * Nkv * ((H + BR_BN - 1) / BR_BN) * 2 >= (1LL << 31)) return fail(BR_ERR_ARG, "batch too large for one backward launch");
+    if (((long long)M * B * Nkv + 7) * 4 * ((H + BR_BN - 1) / BR_BN) >= (1LL << 31)) return fail(BR_ERR_ARG, "batch too large for one backward launch");
     p.dq = dq; p.dk = dk; p.dv = dv;
     p.dq_b = dq_strides[0]; p.dq_h = dq_strides[1]; p.dq_t = dq_strides[2];
     p.dk_b = dk_strides[0]; p.dk_h = dk_strides[1]; p.dk_t = dk_strides[2];
