@@ -47,6 +47,13 @@ def test_pure_host_entry_points():
     assert lib.br_prefill_workspace_bytes_fused(4, 22, 32, 8, 128) == 4 * 44 * 8 * 128 * 130 * 4
     assert lib.br_prefill_workspace_bytes_fused(4, 5, 32, 8, 128) == lib.br_prefill_workspace_bytes(4, 32, 8, 128)
     assert lib.br_prefill_fp8qk_workspace_bytes(4, 32, 8, 128, 4 * 3520) > lib.br_prefill_workspace_bytes(4, 32, 8, 128)
+    # backward: fp32 sums of the query block's dQ rows and of the prefix keys' dK / dV, rounded up to 256 bytes, then one
+    # float per token slot and query head (delta)
+    assert lib.br_prefill_bwd_workspace_bytes(4, 32, 8, 160, 128, 4 * 3520) == 4 * (32 + 16) * 160 * 128 * 4 + 4 * 3520 * 32 * 4
+    assert lib.br_prefill_bwd_workspace_bytes(0, 32, 8, 160, 128, 10) == 0
+    rc = lib.br_prefill_bwd(None, None, None, None, None, None, None, 1, 4, 2, 3, 8, 96, None, None, None, None, None, None,
+                            None, None, None, None, None, None, 1.0, 24, None, 0, None)
+    assert rc == _lib.BR_ERR_ARG and b"head dim" in lib.br_last_error()
     # argument errors come back as codes with a message, before anything touches a device
     rc = lib.br_prefill_fwd(None, None, None, None, None, 1, 4, 2, 3, 8, 96, None, None, None, None, 1.0, 1, None, 0, None)
     assert rc == _lib.BR_ERR_ARG and b"head dim" in lib.br_last_error()
