@@ -167,6 +167,8 @@ def bench_model(args):
     ranker = br.TruncatedRanker(model, layer_idx)
     if not args.hf_rope:
         br.patch_rotary(model)           # the one-pass rotary embedding kernel instead of the model file's eager expression
+    if not args.hf_layer_ops:
+        br.patch_layer_ops(model)        # one-pass RMSNorm and SiLU-gate kernels instead of the model file's eager expressions
     steps = args.steps if args.steps is not None else 10
     warmup = args.warmup if args.warmup is not None else 2
     if args.padded:
@@ -215,7 +217,8 @@ def bench_model(args):
                    "name": "cfg3", "batch": B, "blocks": layout.M, "block_len": layout.H, "valid_tokens": layout.valid_tokens,
                    "padded_tokens": B * S, "unmasked_pairs": pairs_n, "launch": "eager",
                    "token_layout": "padded (B, M, H)" if args.padded else "packed (real tokens only)",
-                   "rotary": "model's eager expression" if args.hf_rope else "one-pass HIP kernel"},
+                   "rotary": "model's eager expression" if args.hf_rope else "one-pass HIP kernel",
+                   "norm_and_gate": "model's eager expressions" if args.hf_layer_ops else "one-pass HIP kernels"},
         "prefill_tok_per_s": layout.valid_tokens / (ms_per_step * 1e-3),
         "attention_ms_per_step": sum(kern_ms),
         "attention_share": sum(kern_ms) / ms_per_step,
@@ -293,6 +296,8 @@ def main():
     ap.add_argument("--backward", action="store_true",
                     help="time the training step of the attention instead: forward that saves the log-sum-exp, then the backward kernels")
     ap.add_argument("--hf-rope", action="store_true", help="cfg3: keep the model file's own rotary embedding (eight elementwise passes per layer)")
+    ap.add_argument("--hf-layer-ops", action="store_true",
+                    help="cfg3: keep the model file's own RMSNorm and SiLU-gate expressions (ten elementwise passes per layer)")
     ap.add_argument("--padded", action="store_true",
                     help="cfg3: feed the reference's padded (B, M, H) batch instead of the packed one")
     ap.add_argument("--calibrate-copy", action="store_true",

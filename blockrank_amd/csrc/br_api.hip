@@ -30,6 +30,9 @@ int br_launch_last_logits(const void* q, const void* k, const int* plan, const i
                           float neg, int dtype, hipStream_t stream);
 
 int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, hipStream_t stream);
+int br_launch_rmsnorm(const void* x, const void* w, void* out, long long rows, int hidden, long long sx, long long so, float eps, int dtype,
+                      int n_cu, hipStream_t stream);
+void br_launch_silu_mul(const void* gate, const void* up, void* out, long long n, int dtype, int n_cu, hipStream_t stream);
 
 namespace {
 
@@ -499,6 +502,36 @@ int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, v
     const long long sc[2] = {cs_strides[0], cs_strides[1]};
     br_launch_rope(q, k, cos, sin, q_out, k_out, B, Nq, Nkv, S, D, sq, sk, sc, dtype, n_cu, static_cast<hipStream_t>(stream));
     return check_launch("rotary embedding launch");
+}
+
+int br_rmsnorm(const void* x, const void* weight, void* out, int64_t rows, int hidden, int64_t x_row_stride, int64_t out_row_stride,
+               float eps, int dtype, void* stream) {
+    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "dtype must be fp32 (0) or bf16 (1)");
+    if (rows < 0 || hidden <= 0) return fail(BR_ERR_ARG, "rows and hidden must be positive");
+    const int per16 = dtype == BR_DTYPE_F32 ? 4 : 8;
+    if (hidden % per16 || x_row_stride % per16 || out_row_stride % per16 || x_row_stride < hidden || out_row_stride < hidden)
+        return fail(BR_ERR_ARG, "hidden size and row strides must be multiples of 16 bytes, rows must not overlap");
+    if (!x || !weight || !out) return fail(BR_ERR_ARG, "null pointer");
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(out)) return fail(BR_ERR_ARG, "x, weight and out must be 16-byte aligned");
+    if (rows == 0) return BR_OK;
+    const int n_cu = n_compute_units();
+    if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
+    if (br_launch_rmsnorm(x, weight, out, rows, hidden, x_row_stride, out_row_stride, eps, dtype, n_cu, static_cast<hipStream_t>(stream)))
+        return fail(BR_ERR_ARG, "hidden size %d too large for the RMSNorm kernel", hidden);
+    return check_launch("RMSNorm launch");
+}
+
+int br_silu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, void* stream) {
+    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "dtype must be fp32 (0) or bf16 (1)");
+    const int per16 = dtype == BR_DTYPE_F32 ? 4 : 8;
+    if (n < 0 || n % per16) return fail(BR_ERR_ARG, "the element count must be a multiple of 16 bytes");
+    if (!gate || !up || !out) return fail(BR_ERR_ARG, "null pointer");
+    if (!aligned16(gate) || !aligned16(up) || !aligned16(out)) return fail(BR_ERR_ARG, "gate, up and out must be 16-byte aligned");
+    if (n == 0) return BR_OK;
+    const int n_cu = n_compute_units();
+    if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
+    br_launch_silu_mul(gate, up, out, n, dtype, n_cu, static_cast<hipStream_t>(stream));
+    return check_launch("SiLU gate launch");
 }
 
 }  // extern "C"

@@ -1,0 +1,96 @@
+"""RMSNorm and the SiLU-gated product of a decoder layer, each in one HIP pass.
+
+The Hugging Face model classes the reference's models are instances of (transformers
+models/mistral/modeling_mistral.py: ``MistralRMSNorm.forward`` and ``MistralMLP.forward``; the same classes in the
+Llama and Qwen2 model files) express them as eight and two elementwise passes over the activations; the
+ranking forward of scripts/eval_attn.py:139-151 runs them in every decoder layer (measured at the Mistral-7B
+shape: 17 % of the GPU time of a forward pass).  ``patch_layer_ops(model)`` gives the model's norm and MLP
+modules a forward that calls the kernels; with gradients enabled, or on tensors the kernels do not take, the
+module's own forward runs as before.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .attention import _DTYPE_CODE, _stream_ptr
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """weight * (x * rsqrt(mean(x^2, -1) + eps)) for x (..., hidden); fp32 arithmetic, the model file's rounding."""
+    assert x.is_cuda and x.dtype in _DTYPE_CODE and weight.dtype == x.dtype, "rms_norm takes bf16 or fp32 device tensors of one dtype"
+    hidden = x.shape[-1]
+    assert weight.shape == (hidden,), "weight must have the size of the last dim"
+    per16 = 16 // x.element_size()
+    x2 = x.reshape(-1, hidden)
+    if x2.stride(-1) != 1 or x2.stride(0) % per16 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    w = weight if weight.is_contiguous() and weight.data_ptr() % 16 == 0 else weight.contiguous()
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        out = torch.empty((x2.shape[0], hidden), dtype=x.dtype, device=x.device)
+        _lib.check(lib.br_rmsnorm(x2.data_ptr(), w.data_ptr(), out.data_ptr(), x2.shape[0], hidden, x2.stride(0), hidden, float(eps),
+                                  _DTYPE_CODE[x.dtype], _stream_ptr(x.device)))
+    return out.view(x.shape)
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up, elementwise, tensors of one shape and dtype (bf16 or fp32)."""
+    assert gate.is_cuda and gate.dtype in _DTYPE_CODE and up.dtype == gate.dtype and up.shape == gate.shape
+    g, u = gate.contiguous(), up.contiguous()
+    lib = _lib.load()
+    with torch.cuda.device(gate.device):
+        out = torch.empty_like(g)
+        _lib.check(lib.br_silu_mul(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _DTYPE_CODE[g.dtype], _stream_ptr(g.device)))
+    return out
+
+
+def _kernel_ok(x: torch.Tensor, *params: torch.Tensor) -> bool:
+    if not x.is_cuda or x.dtype not in _DTYPE_CODE or (x.shape[-1] * x.element_size()) % 16:
+        return False
+    if any(p.dtype != x.dtype for p in params):
+        return False
+    return not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in params)))
+
+
+def patch_layer_ops(model) -> int:
+    """Give every ``*RMSNorm`` module (``weight``, ``variance_epsilon``) and every gated ``*MLP`` module
+    (``gate_proj``, ``up_proj``, ``down_proj``, SiLU activation) of ``model`` a forward that uses the kernels.
+    Returns the number of modules patched; ``unpatch_layer_ops`` restores them."""
+    n = 0
+    for m in model.modules():
+        if "_blockrank_amd_saved_forward" in m.__dict__:
+            continue
+        name = type(m).__name__
+        if name.endswith("RMSNorm") and hasattr(m, "weight") and hasattr(m, "variance_epsilon"):
+            orig = m.forward
+
+            def norm_forward(hidden_states, _m=m, _orig=orig):
+                if not _kernel_ok(hidden_states, _m.weight):
+                    return _orig(hidden_states)
+                return rms_norm(hidden_states, _m.weight, _m.variance_epsilon)
+
+            m.__dict__["_blockrank_amd_saved_forward"] = orig
+            m.forward = norm_forward
+            n += 1
+        elif name.endswith("MLP") and all(hasattr(m, a) for a in ("gate_proj", "up_proj", "down_proj", "act_fn")) and \
+                "silu" in type(m.act_fn).__name__.lower():
+            orig = m.forward
+
+            def mlp_forward(x, _m=m, _orig=orig):
+                if not _kernel_ok(x, _m.gate_proj.weight):
+                    return _orig(x)
+                return _m.down_proj(silu_mul(_m.gate_proj(x), _m.up_proj(x)))
+
+            m.__dict__["_blockrank_amd_saved_forward"] = orig
+            m.forward = mlp_forward
+            n += 1
+    return n
+
+
+def unpatch_layer_ops(model) -> None:
+    for m in model.modules():
+        if "_blockrank_amd_saved_forward" in m.__dict__:
+            del m.__dict__["_blockrank_amd_saved_forward"]
+            if "forward" in m.__dict__:
+                del m.__dict__["forward"]

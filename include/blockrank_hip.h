@@ -229,6 +229,19 @@ int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out,
                    const int64_t* dv_strides, float scale, int64_t token_slots, void* workspace, size_t workspace_bytes,
                    void* stream);
 
+/* ---- the elementwise steps of a decoder layer around the attention, one pass each ----
+ * Both replace methods of the Hugging Face model classes the reference's models are instances of (transformers
+ * models/mistral/modeling_mistral.py: MistralRMSNorm.forward, MistralMLP.forward; the same in the Llama and Qwen2
+ * model files), which the ranking forward of scripts/eval_attn.py:139-151 runs in every decoder layer.
+ *
+ * br_rmsnorm: out[r, :] = weight * (x[r, :] * rsqrt(mean(x[r, :]^2) + eps)), fp32 arithmetic; for bf16 the normalised
+ * value is rounded to bf16 before the multiplication by the weight, as in the model file.  x, out: rows x hidden with
+ * the given row strides (elements); weight: hidden.  dtype 0 fp32, 1 bf16.
+ * br_silu_mul: out = silu(gate) * up over n contiguous elements (silu rounded to the tensor type first). */
+int br_rmsnorm(const void* x, const void* weight, void* out, int64_t rows, int hidden, int64_t x_row_stride, int64_t out_row_stride,
+               float eps, int dtype, void* stream);
+int br_silu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

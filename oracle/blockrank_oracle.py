@@ -34,6 +34,12 @@ How each function is pinned (see tests/test_oracle_*.py):
                                    closed form (angle 0 = identity, pair norms preserved, angle then minus
                                    angle = identity, the vector (1, 0) goes to (cos, sin)) and against
                                    complex multiplication.
+  rms_norm, silu_mul               restate third-party functions the reference calls through the model forward
+                                   (same transformers files): pinned by closed forms - with unit weight and eps = 0
+                                   every output row has mean square 1, scaling a row leaves its output unchanged,
+                                   a constant row c gives sign(c) * weight; silu(0) = 0, silu(g) -> g for large g,
+                                   silu(g) - silu(-g) = g, and against torch.nn.functional.silu / the published formula
+                                   written with torch ops.
 No golden vectors exist in the reference (it ships no tests); none of the functions above needed
 an import of the reference to be pinned, so the reference was only read, never run.
 """
@@ -426,3 +432,18 @@ def rotary_embedding(x: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndar
     h = x.shape[-1] // 2
     rot = np.concatenate([-x[..., h:], x[..., :h]], axis=-1)
     return x * c + rot * s_
+
+
+def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """weight * x / sqrt(mean(x^2, -1) + eps) in float64: the RMSNorm of the Hugging Face decoder classes
+    (transformers models/mistral/modeling_mistral.py, MistralRMSNorm.forward; the same class in the Llama and
+    Qwen2 files), which the reference reaches through the model forward of scripts/eval_attn.py:139-151."""
+    x = np.asarray(x, dtype=np.float64)
+    return np.asarray(weight, dtype=np.float64) * x / np.sqrt((x * x).mean(axis=-1, keepdims=True) + eps)
+
+
+def silu_mul(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """silu(gate) * up with silu(g) = g / (1 + exp(-g)) in float64: the gated product of MistralMLP.forward
+    (same model files)."""
+    g = np.asarray(gate, dtype=np.float64)
+    return g / (1.0 + np.exp(-g)) * np.asarray(up, dtype=np.float64)
