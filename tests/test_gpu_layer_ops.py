@@ -57,11 +57,12 @@ def test_silu_mul(dtype):
     assert err.mean() <= ref_err.mean() * 1.5 + 1e-9          # (fp32: both are at the last bit; the summation order differs)
 
 
-def test_patched_model_matches_unpatched():
+@pytest.mark.parametrize("kind", ["mistral", "qwen2"])
+def test_patched_model_matches_unpatched(kind):
     from tests.test_gpu_hf_model import build
     from blockrank_amd import synthetic
     br.register_blockrank_attention()
-    model = build("mistral", torch.bfloat16)
+    model = build(kind, torch.bfloat16)
     model.set_attn_implementation("sdpa_blockrank")
     lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
     ids = torch.randint(0, 512, (lay.B, lay.S), generator=torch.Generator().manual_seed(1)).to(DEV)
