@@ -9,7 +9,7 @@ followed by the fused per-document score extraction.  The request plan (block ta
 built once per forward pass by the mask hook and shared by every layer, so it is built outside the
 timed region and its cost is reported separately (``plan_build_ms``).
 
-``--workload cfg3`` is the end-to-end case instead (BASELINE configs[2]): a random-initialised
+``--workload cfg3`` is the end-to-end case instead: a random-initialised
 Mistral-7B-shaped decoder run by the layer-truncated ranking driver (layers 0..19 in full, of layer 20
 only what the scores need), B=8; its line reports requests/s of the whole forward and, from HIP events
 around each layer's attention kernel, that kernel's roofline fraction at this layout.
@@ -44,13 +44,13 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 def workloads():
     from blockrank_amd import synthetic
     return {
-        # BASELINE configs[1]: the configuration the headline metric is quoted on
+        # the configuration the headline metric is quoted on
         "cfg2": dict(desc="Mistral-7B-shaped attention layer, B=4, 32q/8kv heads, D=128, 64-token prefix + 20 docs x 160 + 32-token query (3296 tokens/seq), bf16, proj+RoPE inputs",
                      layout=lambda: synthetic.uniform_layout(4, 64, 20, 160, 32), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
-        # BASELINE configs[3]: long list
+        # long document list
         "cfg4": dict(desc="Mistral-7B attention shapes, B=1, 64-token prefix + 100 docs U[64,384] + 48-token query, bf16",
                      layout=lambda: synthetic.random_layout(1, 64, 100, 64, 384, 48, seed=0), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
-        # BASELINE configs[4] shapes with bf16 QK^T (the fp8 variant is not built)
+        # Qwen2.5-7B head layout and a long-tailed document length distribution (bf16; --qk-fp8 computes Q K^T in fp8)
         "cfg5shape": dict(desc="Qwen2.5-7B attention shapes, B=4, 28q/4kv heads, D=128, 32-token prefix + 50 lognormal docs + 24-token query, bf16",
                           layout=lambda: synthetic.lognormal_layout(4, 32, 50, 120, 0.6, 16, 512, 24, seed=0), Nq=28, Nkv=4, D=128, hidden=3584, dtype=torch.bfloat16),
         "cfg2_b1": dict(desc="cfg2 with B=1", layout=lambda: synthetic.uniform_layout(1, 64, 20, 160, 32), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
@@ -61,7 +61,7 @@ def workloads():
         # the headline layout with eight query heads per kv head (Llama-3-70B-like grouping)
         "cfg2g8": dict(desc="cfg2 layout with 32q/4kv heads (8 per group), D=128, bf16", layout=lambda: synthetic.uniform_layout(4, 64, 20, 160, 32),
                        Nq=32, Nkv=4, D=128, hidden=None, dtype=torch.bfloat16),
-        # BASELINE configs[0]: the reference's CPU-runnable case
+        # the small fp32 case that also runs on a CPU in seconds
         "cfg1": dict(desc="fp32, B=1, 8q/2kv heads, D=64, 32-token prefix + 8 docs x 64 + 16-token query", layout=lambda: synthetic.uniform_layout(1, 32, 8, 64, 16),
                      Nq=8, Nkv=2, D=64, hidden=None, dtype=torch.float32),
     }

@@ -400,7 +400,7 @@ def eval_labels(valid: np.ndarray) -> np.ndarray:
 
 def quantize_fp8_e4m3(x: torch.Tensor, valid: torch.Tensor) -> torch.Tensor:
     """Per-(sequence, head) absmax quantisation to fp8 e4m3 and back, as the fp8 Q K^T variant defines
-    it (no reference counterpart; BASELINE config 5): scale = max |x| over the sequence's real tokens
+    it (no reference counterpart; the Qwen2.5-7B-shaped benchmark configuration): scale = max |x| over the sequence's real tokens
     / 448; x / scale rounded to the nearest e4m3 value (torch.float8_e4m3fn, round to nearest even,
     the same format the gfx950 conversion instruction produces); returned dequantised, in float32.
     x (B, heads, S, D); valid (B, M, H) with M*H = S.  Pinned by: values that are exactly representable

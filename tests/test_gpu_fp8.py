@@ -1,4 +1,4 @@
-"""Q K^T in fp8 e4m3 with per-head absmax scales, P V in bf16 (BASELINE config 5, Qwen2.5-7B attention
+"""Q K^T in fp8 e4m3 with per-head absmax scales, P V in bf16 (the benchmark configuration with Qwen2.5-7B attention
 shapes: 28 query heads / 4 kv heads, D = 128).  Two checks:
   * against the oracle fed with the same quantised Q and K (oracle.quantize_fp8_e4m3): the kernel's own
     arithmetic, to the usual bf16 bar (outputs 2e-2 max-abs, scores 1e-3 relative);
@@ -48,7 +48,7 @@ def test_fp8_kernel_matches_oracle_on_quantised_inputs(Nq, Nkv, kind):
 
 
 def test_config5_scores_against_fp32_oracle():
-    # BASELINE config 5 at full size: B=4, 50 lognormal documents, projection + RoPE inputs
+    # that configuration at full size: B=4, 50 lognormal documents, projection + RoPE inputs
     lay = synthetic.lognormal_layout(4, 32, 50, 120, 0.6, 16, 512, 24, seed=0)
     q, k, v, out, scores, scale = _run(lay, 28, 4, 0, hidden=3584)
     want = oracle_doc_scores(q, k, lay, scale)                    # unquantised
