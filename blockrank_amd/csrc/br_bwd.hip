@@ -201,6 +201,11 @@ struct Bwd {
         Tile cur, nxt;
         bool have = next_tile(cur);
         if (have) load_tile(cur);
+        // Everything requested so far (Q, dO, O, the first tile) is needed before the first product anyway: wait here,
+        // so that the loop is entered with no load pending.  Otherwise the compiler's wait-count bookkeeping keeps
+        // partial waits in front of every use of Q and dO inside the loop, and those waits count the tile requested
+        // ahead - the look-ahead would wait for itself.
+        __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0); expcnt and lgkmcnt not waited for
         while (have) {
             const bool self = cur.self;
             const int nvalid = cur.nvalid, key0 = cur.key0;
@@ -398,6 +403,11 @@ struct Bwd {
             float stat_c = 0.f, stat_n = 0.f;
             bool have = next_step(cur);
             if (have && has_work(cur)) load_step(cur, rv, stat_c);
+            // Wait for the first step's rows here.  Entering the loop with loads still pending makes the compiler's
+            // wait-count bookkeeping treat the current rows as "loaded a few requests ago" in every iteration: it
+            // then puts partial waits in front of each use, and those waits count the rows requested ahead for
+            // the next step - the look-ahead would wait for itself.
+            __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0); expcnt and lgkmcnt not waited for
             while (have) {
                 const bool have_next = next_step(nxt);
                 const bool work = has_work(cur);
