@@ -169,6 +169,7 @@ def bench_model(args):
         br.patch_rotary(model)           # the one-pass rotary embedding kernel instead of the model file's eager expression
     if not args.hf_layer_ops:
         br.patch_layer_ops(model)        # one-pass RMSNorm and SiLU-gate kernels instead of the model file's eager expressions
+        br.patch_qkv(model)              # one GEMM for the Q, K and V projections of a layer
     steps = args.steps if args.steps is not None else 10
     warmup = args.warmup if args.warmup is not None else 2
     if args.padded:
@@ -218,7 +219,8 @@ def bench_model(args):
                    "padded_tokens": B * S, "unmasked_pairs": pairs_n, "launch": "eager",
                    "token_layout": "padded (B, M, H)" if args.padded else "packed (real tokens only)",
                    "rotary": "model's eager expression" if args.hf_rope else "one-pass HIP kernel",
-                   "norm_and_gate": "model's eager expressions" if args.hf_layer_ops else "one-pass HIP kernels"},
+                   "norm_and_gate": "model's eager expressions" if args.hf_layer_ops else "one-pass HIP kernels",
+                   "qkv_projection": "three GEMMs" if args.hf_layer_ops else "one stacked GEMM"},
         "prefill_tok_per_s": layout.valid_tokens / (ms_per_step * 1e-3),
         "attention_ms_per_step": sum(kern_ms),
         "attention_share": sum(kern_ms) / ms_per_step,

@@ -27,7 +27,7 @@ from .losses import compute_auxiliary_attention_loss, rank_documents
 from .ranker import TruncatedRanker
 from .collate import block_icr_collate_packed, pack_padded_batch
 from .rope import apply_rotary_pos_emb, patch_rotary, unpatch_rotary
-from .layer_ops import patch_layer_ops, rms_norm, silu_mul, unpatch_layer_ops
+from .layer_ops import patch_layer_ops, patch_qkv, rms_norm, silu_mul, unpatch_layer_ops, unpatch_qkv
 
 __all__ = [
     "apply_rotary_pos_emb",
@@ -37,6 +37,8 @@ __all__ = [
     "silu_mul",
     "patch_layer_ops",
     "unpatch_layer_ops",
+    "patch_qkv",
+    "unpatch_qkv",
     "BlockMask",
     "LastBlockScores",
     "blockrank_attention",

@@ -83,3 +83,36 @@ def test_patched_model_matches_unpatched(kind):
     out = model(**kw).hidden_states[-1]
     assert out.requires_grad
     br.unpatch_layer_ops(model)
+
+
+@pytest.mark.parametrize("kind", ["mistral", "qwen2"])
+def test_stacked_qkv_projection(kind):
+    """patch_qkv: one GEMM for the three projections of a decoder layer.  A GEMM over the stacked weight may round its
+    sums in another order than three separate ones, so hidden states are compared to the bf16 bar; the ranking path
+    (TruncatedRanker, which projects K of all tokens and Q of the query block separately at the scoring layer) must
+    keep working on the patched model."""
+    from tests.test_gpu_hf_model import build
+    from blockrank_amd import synthetic
+    br.register_blockrank_attention()
+    model = build(kind, torch.bfloat16)          # qwen2 has projection biases
+    model.set_attn_implementation("sdpa_blockrank")
+    lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
+    lay.labels[:] = -100
+    lay.labels[:, -2:] = 7
+    ids = torch.randint(0, 512, (lay.B, lay.S), generator=torch.Generator().manual_seed(1)).to(DEV)
+    pos, valid, labels = lay.position_ids.to(DEV), lay.valid.to(DEV), lay.labels.to(DEV)
+    kw = dict(input_ids=ids, position_ids=pos, attention_mask=valid, output_hidden_states=True, use_cache=False)
+    ranker = br.TruncatedRanker(model, 1)
+    with torch.no_grad():
+        ref = model(**kw).hidden_states[-1].float()
+        ref_scores = ranker(ids, valid, pos, labels=labels)
+        assert br.patch_qkv(model) == 3
+        got = model(**kw).hidden_states[-1].float()
+        got_scores = ranker(ids, valid, pos, labels=labels)
+        br.unpatch_qkv(model)
+        again = model(**kw).hidden_states[-1].float()
+    rows = valid.reshape(lay.B, lay.S)
+    assert torch.equal(again, ref), "unpatching restores the model's own projections"
+    err = (got[rows] - ref[rows]).abs().max().item()
+    assert err <= 3e-2 * max(1.0, ref[rows].abs().max().item()), f"hidden state differs by {err}"
+    torch.testing.assert_close(got_scores, ref_scores, rtol=2e-2, atol=1e-3)
