@@ -638,13 +638,8 @@ __global__ __launch_bounds__(256) void br_bwd_dq_finish_kernel(BrBwdParams p) {
 
 template <int D, int MAXW>
 int launch_dq(const BrBwdParams& p, int NW, hipStream_t stream) {
-    const int lds = Bwd<D>::dqLdsBytes;
-    static bool armed = false;
-    if (!armed) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&br_bwd_dq_kernel<D, MAXW>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-            return -2;
-        armed = true;
-    }
+    constexpr int lds = Bwd<D>::dqLdsBytes;
+    static_assert(lds <= 65536, "dynamic LDS above 64 KiB would need hipFuncSetAttribute");
     hipLaunchKernelGGL((br_bwd_dq_kernel<D, MAXW>), dim3(p.max_items * p.geom.NHG), dim3(NW * 64), lds, stream, p);
     return 0;
 }
@@ -655,12 +650,8 @@ int launch_all(const BrBwdParams& p, int NW, int n_cu, hipStream_t stream) {
     hipLaunchKernelGGL(br_fill_zero_kernel, dim3(n_cu * 4), dim3(256), 0, stream, reinterpret_cast<uint4*>(p.dq32), n16);
     const int rc = NW <= 4 ? launch_dq<D, 4>(p, NW, stream) : launch_dq<D, 8>(p, NW, stream);
     if (rc) return rc;
-    const int lds = Bwd<D>::dkvLdsBytes;
-    static bool armed = false;
-    if (!armed) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&br_bwd_dkv_kernel<D>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
-        armed = true;
-    }
+    constexpr int lds = Bwd<D>::dkvLdsBytes;
+    static_assert(lds <= 65536, "dynamic LDS above 64 KiB would need hipFuncSetAttribute");
     const int KT = (p.H + BR_BN - 1) / BR_BN;
     hipLaunchKernelGGL((br_bwd_dkv_kernel<D>), dim3((p.M * p.B * p.Nkv + 7) / 8 * 8 * 4 * KT), dim3(128), lds, stream, p);
     hipLaunchKernelGGL((br_bwd_dq_finish_kernel<D>), dim3(n_cu * 4), dim3(256), 0, stream, p);
@@ -669,7 +660,7 @@ int launch_all(const BrBwdParams& p, int NW, int n_cu, hipStream_t stream) {
 
 }  // namespace
 
-// Returns 0 on success, -1 if D has no instance, -2 if a kernel's LDS size could not be set.
+// Returns 0 on success, -1 if D has no instance.
 int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, hipStream_t stream) {
     if (D == 128) return launch_all<128>(p, NW, n_cu, stream);
     if (D == 64) return launch_all<64>(p, NW, n_cu, stream);

@@ -11,11 +11,13 @@ void launch(const BrPrefillParams& p, int grid, hipStream_t stream) {
 
 template <int D>
 int launch_resident(const BrPrefillParams& p, int n_cu, hipStream_t stream) {
-    static bool armed = false;     // (per process; the attribute is set for the current device's function)
+    static bool armed[64] = {};    // per device: the attribute belongs to the function as loaded on that device
     const void* fn = reinterpret_cast<const void*>(&br_prefill_resident_kernel<D>);
-    if (!armed) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return -1;
+    if (dev < 0 || dev >= 64 || !armed[dev]) {
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, Resident<D>::kLdsBytes) != hipSuccess) return -1;
-        armed = true;
+        if (dev >= 0 && dev < 64) armed[dev] = true;
     }
     hipLaunchKernelGGL((br_prefill_resident_kernel<D>), dim3(n_cu), dim3(512), Resident<D>::kLdsBytes, stream, p);
     return 0;
