@@ -36,6 +36,7 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -384,7 +385,7 @@ struct Prefill {
     // variant is one straight-line block with the LDS operand reads issued ahead of their use.
     template <int NKB, bool MASK>
     static __device__ inline void compute_tile(const char* stage, const Lane& L, const Frag (&qf)[D / 16], f32x16 (&o)[D / 32],
-                                               float& m_run, float& l_run, float scale_log2, int lim, int lh, float& psum_out) {
+                                               float& m_run, float& l_run, float& lt_run, float scale_log2, int lim, int lh, float& psum_out) {
         constexpr int NC = D / 16, ND = D / 32, NR = NKB * NC;
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         f32x16 s[NKB];
@@ -431,13 +432,19 @@ struct Prefill {
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_sub);
             m_run = m_new;
             l_run *= alpha;
+            lt_run *= alpha;
 #pragma unroll
             for (int d = 0; d < ND; ++d)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
         }
         const float m_sub = m_run == -INFINITY ? 0.f : m_run;
-        float psum = 0.f;
+        // Two sums of the probabilities: the exact one (log-sum-exp, score partials) and the sum of the values
+        // as rounded to bf16 for the P V product.  The output is normalised by the second: numerator and
+        // denominator then carry the same rounding, and a row whose mass sits on one key reproduces that key's
+        // V row exactly instead of V * (rounded p / p).
+        float psum = 0.f, psum_t = 0.f;
+        const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
         bf16x8 pf[2 * NKB];
 #pragma unroll
         for (int c2 = 0; c2 < 2 * NKB; ++c2) {
@@ -448,8 +455,13 @@ struct Prefill {
                 psum += t[e];
             }
             pf[c2] = __builtin_convertvector(t, bf16x8);
+            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 0, 1), ones2, psum_t, false);
+            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 2, 3), ones2, psum_t, false);
+            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 4, 5), ones2, psum_t, false);
+            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 6, 7), ones2, psum_t, false);
         }
         l_run += psum;
+        lt_run += psum_t;
         psum_out = psum;
 #pragma unroll
         for (int c2 = 0; c2 < 2 * NKB; ++c2) {
@@ -574,7 +586,7 @@ struct Prefill {
         for (int d = 0; d < D / 32; ++d)
 #pragma unroll
             for (int v = 0; v < 16; ++v) o[d][v] = 0.f;
-        float m_run = -INFINITY, l_run = 0.f;
+        float m_run = -INFINITY, l_run = 0.f, lt_run = 0.f;
 
         vm_wait_all();
         // tell the compiler the Q fragments are in registers now: otherwise it would put its own
@@ -614,13 +626,13 @@ struct Prefill {
             const bool need_mask = (v_nvalid < nkb * 32) || (c_self && key0 + nkb * 32 - 1 > row0);
             float psum = 0.f;
             if (nkb == 2 && !need_mask) {
-                compute_tile<2, false>(stage, L, qf, o, m_run, l_run, sc2, 0, lh, psum);
+                compute_tile<2, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, 0, lh, psum);
             } else if (nkb > 0) {
                 const int lim_causal = c_self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
                 const int lim = v_nvalid < lim_causal ? v_nvalid : lim_causal;
-                if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, sc2, lim, lh, psum);
-                else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, sc2, lim, lh, psum);
-                else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, sc2, lim, lh, psum);
+                if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
             }
             // Score partials: this tile's probability mass (against the running max) for the query block's
             // last rows, per head - everything the per-document scores need, with no second pass over K.
@@ -647,7 +659,8 @@ struct Prefill {
         // to the top of the item where they would have to be spilled across the key loop)
         int lane_e = lane;
         asm volatile("" : "+v"(lane_e));
-        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        const float l_tot = l_run + __shfl_xor(l_run, 32);       // exact sum: log-sum-exp
+        const float lt_tot = lt_run + __shfl_xor(lt_run, 32);    // sum of the rounded probabilities: normalises the output
         if (it.slot >= 0) {
             if (row0 + ln < len_m) {
                 const long long slot = ((long long)b * p.slots + it.slot) * ge.NHG + hg;
@@ -662,14 +675,14 @@ struct Prefill {
                     }
                 if (lh == 0) {
                     p.part_ml[prow * 2] = m_run;
-                    p.part_ml[prow * 2 + 1] = l_tot;
+                    p.part_ml[prow * 2 + 1] = lt_tot;
                 }
             }
         } else {
             // the last loop iteration ended with a barrier, so the K/V buffers are free: transpose
             // through LDS so that every output row is written as full 16-byte pieces
             __bf16* Es = reinterpret_cast<__bf16*>(smem + wave * SM::eBytesPerWave);
-            const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;
+            const float inv = lt_tot > 0.f ? __builtin_amdgcn_rcpf(lt_tot) : 0.f;
             if (p.lse != nullptr && lane_e < 32 && row0 + lane_e < len_m)
                 p.lse[(long long)b * p.lse_b + (long long)head * p.lse_h + qtok0 + row0 + lane_e] = m_run + __builtin_amdgcn_logf(l_tot);
             if (rb_active) {
@@ -810,7 +823,7 @@ struct Resident {
         for (int d = 0; d < D / 32; ++d)
 #pragma unroll
             for (int v = 0; v < 16; ++v) o[d][v] = 0.f;
-        float m_run = -INFINITY, l_run = 0.f;
+        float m_run = -INFINITY, l_run = 0.f, lt_run = 0.f;
 
         for (int f = f_lo; f < f_hi; ++f) {
             const char* stage = smem + f * SM::stageBytes;
@@ -831,13 +844,13 @@ struct Resident {
             const bool need_mask = (v_nvalid < nkb * 32) || (c_self && v_key0 + nkb * 32 - 1 > row0);
             float psum = 0.f;
             if (nkb == 2 && !need_mask) {
-                PF::template compute_tile<2, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, 0, lh, psum);
+                PF::template compute_tile<2, false>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, 0, lh, psum);
             } else if (nkb > 0) {
                 const int lim_causal = c_self ? row0 + ln - v_key0 + 1 : BR_BN;
                 const int lim = v_nvalid < lim_causal ? v_nvalid : lim_causal;
-                if (nkb == 2) PF::template compute_tile<2, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
-                else if (need_mask) PF::template compute_tile<1, true>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
-                else PF::template compute_tile<1, false>(stage, L, qf, o, m_run, l_run, p.scale_log2, lim, lh, psum);
+                if (nkb == 2) PF::template compute_tile<2, true>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, lim, lh, psum);
+                else if (need_mask) PF::template compute_tile<1, true>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, lim, lh, psum);
+                else PF::template compute_tile<1, false>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, lim, lh, psum);
             }
             if (scores) {
                 // this tile's probability mass (against the running max) for the query block's last rows
@@ -863,7 +876,8 @@ struct Resident {
         int lane_e = lane;
         asm volatile("" : "+v"(lane_e));
         const int ln_e = lane_e & 31, lh_e = lane_e >> 5;
-        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        const float l_tot = lt_run + __shfl_xor(lt_run, 32);     // sum of the rounded probabilities (see compute_tile)
+        (void)l_run;
         const bool ok = row0 + ln_e < q_len;
         if (slot >= 0) {
             if (ok) {

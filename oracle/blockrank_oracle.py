@@ -75,8 +75,10 @@ def additive_mask(valid: torch.Tensor, dtype: torch.dtype = torch.float32) -> to
     return out
 
 
-def allowed(valid: np.ndarray) -> np.ndarray:
-    """(B, M, H) bool -> (B, S, S) bool, the element-wise predicate "query token may see key token".
+def allowed(valid: np.ndarray, first_row: int = 0) -> np.ndarray:
+    """(B, M, H) bool -> (B, S - first_row, S) bool, the element-wise predicate "query token may see key
+    token" for the query tokens first_row .. S-1 (all of them by default; the score rows are the last few,
+    and a long request's full S x S table would be gigabytes).
 
     Follows blockrank_mask_fn, blockrank_std_attention.py:344-399: both tokens valid, and
       block 0      : same block, causal
@@ -88,8 +90,8 @@ def allowed(valid: np.ndarray) -> np.ndarray:
     S = M * H
     idx = np.arange(S)
     blk, pos = idx // H, idx % H
-    qb, kb = blk[:, None], blk[None, :]
-    qp, kp = pos[:, None], pos[None, :]
+    qb, kb = blk[first_row:, None], blk[None, :]
+    qp, kp = pos[first_row:, None], pos[None, :]
     same = qb == kb
     causal = qp >= kp
     is0 = qb == 0
@@ -100,7 +102,7 @@ def allowed(valid: np.ndarray) -> np.ndarray:
     patl = last & ((same & causal) | (~same & (kb < qb)))
     pattern = pat0 | patm | patl
     flat = valid.reshape(B, S)
-    return flat[:, :, None] & flat[:, None, :] & pattern[None]
+    return flat[:, first_row:, None] & flat[:, None, :] & pattern[None]
 
 
 def segment_masks(mask5: torch.Tensor) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
@@ -301,21 +303,21 @@ def sdpa_blockrank_forward(
 def last_block_logits(q, k, valid, scale: float, num_last_queries: int = 16, neg: float = None) -> np.ndarray:
     """Closed form of s_last in float64: scale*q.k + (0 if allowed else NEG) for the last R rows of
     the last block against all S keys.  (blockrank_std_attention.py:233,259 / :639-645.)"""
-    q = np.asarray(q, dtype=np.float64)
-    k = np.asarray(k, dtype=np.float64)
     valid = np.asarray(valid, dtype=bool)
-    B, Nq, S, D = q.shape
-    Nkv = k.shape[1]
-    G = Nq // Nkv
+    B, Nq, S, D = np.shape(q)
     _, M, H = valid.shape
     R = num_last_queries if H >= num_last_queries else H
+    q = np.asarray(np.asarray(q)[:, :, S - R:], dtype=np.float64)      # only these rows are used
+    k = np.asarray(k, dtype=np.float64)
+    Nkv = k.shape[1]
+    G = Nq // Nkv
     if neg is None:
         neg = neg_value(torch.float32)
-    ok = allowed(valid)[:, S - R:, :]                         # (B,R,S)
+    ok = allowed(valid, first_row=S - R)                      # (B,R,S)
     out = np.empty((B, Nq, R, S))
     for b in range(B):
         for n in range(Nq):
-            s = scale * (q[b, n, S - R:] @ k[b, n // G].T)
+            s = scale * (q[b, n] @ k[b, n // G].T)
             out[b, n] = s + np.where(ok[b], 0.0, neg)
     return out
 
