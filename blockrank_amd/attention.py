@@ -302,9 +302,10 @@ def blockrank_attention(
     score partials of the query block's last score_rows positions, and the call returns
     (out, partials); ``doc_scores_from_partials`` turns them into per-document scores.
 
-    qk_fp8 (bf16 inputs, head dim 128): Q K^T is computed in fp8 e4m3 with per-(sequence, head) absmax
-    scales, P V stays bf16 - the reduced-precision variant for ranking (scores stay within 5e-3
-    relative of the fp32 result)."""
+    qk_fp8 (bf16 inputs, head dim 128): Q K^T of the prefix and document blocks is computed in fp8 e4m3
+    (K with one power-of-two scale per (sequence, kv head), every query row with its own), P V
+    stays bf16; the query block's rows, from which the scores are read, are computed in bf16 - the
+    reduced-precision variant for ranking (scores as accurate as the bf16 kernel's)."""
     if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
         block_mask = BlockMask(block_mask, query.dtype)
     bm = _as_block_mask(block_mask)

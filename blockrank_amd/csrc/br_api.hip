@@ -18,9 +18,8 @@ int br_launch_doc_scores(const void* q, const void* k, const int* plan, const in
                          int R, int T, float scale, float out_scale, int dtype, hipStream_t stream);
 int br_launch_prefill_fp8qk(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                             hipEvent_t ev_start, hipEvent_t ev_stop);
-void br_launch_quantize_fp8(const void* q, const void* k, const int* plan, void* q8, void* k8, unsigned* amax, float* scales,
-                            const long long* sq, const long long* sk, long long q8_b, long long q8_h, long long k8_b, long long k8_h,
-                            int B, int Nq, int Nkv, int M, int H, int D, hipStream_t stream);
+void br_launch_quantize_fp8(const void* k, const int* plan, void* k8, unsigned* amax, float* scales, const long long* sk,
+                            long long k8_b, long long k8_h, int B, int Nkv, int M, int H, int D, hipStream_t stream);
 int br_launch_rope(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
                    int D, const long long* sq, const long long* sk, const long long* sc, int dtype, int n_cu, hipStream_t stream);
 int br_launch_doc_scores_tiles(const float* part, const int* plan, const int* rows, float* scores, float* probs, int B, int Nq,
@@ -199,7 +198,7 @@ static size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int64_t tokens) {
     const size_t base = br_prefill_workspace_bytes(B, Nq, Nkv, D);
     if (base == 0 || tokens <= 0) return 0;
-    return up256(base) + up256((size_t)Nq * tokens * D) + up256((size_t)Nkv * tokens * D) + 2 * up256((size_t)B * (Nq + Nkv) * 4);
+    return up256(base) + up256((size_t)Nkv * tokens * D) + 2 * up256((size_t)B * Nkv * 4);
 }
 
 // fp8_tokens > 0: Q K^T in fp8 (inputs bf16, quantised into the workspace first); it is the length of the
@@ -267,6 +266,8 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     p.score_part = score_part;
     p.score_R = score_part ? score_rows : 0;
     p.qk_scales = nullptr;
+    p.k8 = nullptr;
+    p.k8_b = p.k8_h = 0;
     p.lse = lse;
     p.lse_b = lse ? lse_strides[0] : 0;
     p.lse_h = lse ? lse_strides[1] : 0;
@@ -277,27 +278,21 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     hipEvent_t e0 = static_cast<hipEvent_t>(ev_start), e1 = static_cast<hipEvent_t>(ev_stop);
     int lrc;
     if (fp8_tokens > 0) {
-        const bool packed = q_strides[0] == 0;
-        const long long stot = packed ? fp8_tokens : fp8_tokens / B;        // tokens per batch entry of q8/k8
+        const bool packed = k_strides[0] == 0;
+        const long long stot = packed ? fp8_tokens : fp8_tokens / B;        // tokens per batch entry of k8
+        const long long k8_h = stot * D;
+        const long long k8_b = packed ? 0 : (long long)Nkv * k8_h;
+        if (k8_b >= (1LL << 32) || k8_h >= (1LL << 32)) return fail(BR_ERR_ARG, "fp8 staging strides must be below 2^32 bytes");
         char* w = static_cast<char*>(workspace) + up256(br_prefill_workspace_bytes(B, Nq, Nkv, D));
-        void* q8 = w;
-        w += up256((size_t)Nq * fp8_tokens * D);
         void* k8 = w;
         w += up256((size_t)Nkv * fp8_tokens * D);
         unsigned* amax = reinterpret_cast<unsigned*>(w);
-        w += up256((size_t)B * (Nq + Nkv) * 4);
+        w += up256((size_t)B * Nkv * 4);
         float* scales = reinterpret_cast<float*>(w);
-        const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]}, sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
-        const long long q8_h = stot * D, k8_h = stot * D;
-        const long long q8_b = packed ? 0 : (long long)Nq * q8_h, k8_b = packed ? 0 : (long long)Nkv * k8_h;
-        br_launch_quantize_fp8(q, k, plan, q8, k8, amax, scales, sq, sk, q8_b, q8_h, k8_b, k8_h, B, Nq, Nkv, M, H, D, s);
-        p.q = q8; p.k = k8;
-        p.sq_b = q8_b; p.sq_h = q8_h; p.sq_t = D;
-        p.sk_b = k8_b; p.sk_h = k8_h; p.sk_t = D;
-        if (q8_b >= (1LL << 31) || q8_h >= (1LL << 31) || k8_b >= (1LL << 31) || k8_h >= (1LL << 31))
-            return fail(BR_ERR_ARG, "fp8 staging strides must be below 2^31 elements");
-        p.q32_b = (unsigned)q8_b; p.q32_h = (unsigned)q8_h; p.q32_t = (unsigned)D;
-        p.k32_b = (unsigned)k8_b; p.k32_h = (unsigned)k8_h; p.k32_t = (unsigned)D;
+        const long long sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
+        br_launch_quantize_fp8(k, plan, k8, amax, scales, sk, k8_b, k8_h, B, Nkv, M, H, D, s);
+        p.k8 = k8;
+        p.k8_b = (unsigned)k8_b; p.k8_h = (unsigned)k8_h;
         p.qk_scales = scales;
         lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1);
     } else {

@@ -280,9 +280,12 @@ struct BrPrefillParams {
     // key tile, in the order of the sequence's tile descriptors.  Null: not wanted.
     float* score_part;
     int score_R;
-    // fp8 Q/K variant: q and k then point at e4m3 tensors (strides in elements = bytes) and qk_scales
-    // holds the dequantisation scales, [B][Nq] for Q followed by [B][Nkv] for K.  Null otherwise.
+    // fp8 Q K^T variant: k8 is the e4m3 copy of K ((batch, head) strides k8_b, k8_h in bytes, token stride D) and
+    // qk_scales its dequantisation scales (powers of two), [B][Nkv] (Q is converted in registers by the attention
+    // kernel, one scale per query row).  Null otherwise.
     const float* qk_scales;
+    const void* k8;
+    unsigned k8_b, k8_h;
     // 0: every sequence goes through the streaming kernel; 1: the plan's second view, in which the
     // fused sequences are left to the resident kernel
     int queue_view;

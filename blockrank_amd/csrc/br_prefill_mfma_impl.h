@@ -42,6 +42,7 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 // F8: K (and Q) are fp8 e4m3 (one byte per element, dequantisation scales folded into the softmax
@@ -50,7 +51,10 @@ template <int D, bool F8>
 struct Smem {
     static constexpr int rowB = D * 2;                     // bytes per V row (and per bf16 K row)
     static constexpr int rowKB = F8 ? D : D * 2;           // bytes per K row
-    static constexpr int kBytes = BR_BN * rowKB;
+    static constexpr int kBytes = BR_BN * rowB;            // room of the K tile (an fp8 tile fills half of it): the V tile
+                                                           // sits at the same offset whatever the K element type, so that
+                                                           // items of both kinds can follow each other in one kernel and
+                                                           // the V rows never hold anything but bf16 V data
     static constexpr int vBytes = BR_BN * rowB;
     static constexpr int stageBytes = kBytes + vBytes;     // K tile then V tile
     static constexpr int eRow = D + 8;                     // epilogue tile: [32 rows][eRow] per wave
@@ -242,6 +246,18 @@ struct BrPrefetch {
     }
 };
 
+// Power-of-two quantisation scale of a group whose largest magnitude is amax: 2^(floor(log2(amax)) - 7), which
+// puts that magnitude into [128, 256) of e4m3's range (up to 448), and its inverse.  Multiplying by a power of two
+// is exact, so every implementation of the quantiser rounds the same values the same way.  A group whose maximum
+// is below 2^-119 (or not a number) counts as zero: both results are 0.
+__device__ inline void br_pow2_scale(float amax, float& scale, float& inv) {
+    const unsigned eb = __float_as_uint(fminf(amax, 3.0e38f)) & 0x7f800000u;
+    const bool ok = eb >= (8u << 23);
+    const unsigned sb = eb - (7u << 23);
+    scale = ok ? __uint_as_float(sb) : 0.f;
+    inv = ok ? __uint_as_float((254u << 23) - sb) : 0.f;
+}
+
 typedef long k8x8;   // eight fp8 values: one MFMA operand of v_mfma_f32_32x32x16_fp8_fp8
 
 template <bool F8> struct QKFrag { typedef bf16x8 type; };
@@ -285,7 +301,7 @@ struct Prefill {
             const int slot = (wave + NW * j) * 64 + lane;
             const int prow = slot / CPRK, cp = slot - prow * CPRK;
             const int kkey = (prow & 32) | swap23(prow & 31);
-            L.koff[j] = kkey * (int)p.k32_t * ESZ + ((cp ^ (prow & (CPRK < 8 ? CPRK - 1 : 7))) << 4);
+            L.koff[j] = kkey * (F8 ? D : (int)p.k32_t * 2) + ((cp ^ (prow & (CPRK < 8 ? CPRK - 1 : 7))) << 4);
         }
 #pragma unroll
         for (int j = 0; j < JO; ++j) {
@@ -353,6 +369,24 @@ struct Prefill {
                 }
             }
         }
+    }
+
+    // Eight bf16 values times inv (the inverse of their row's power-of-two scale) as eight e4m3 values, in the
+    // element order of the input (round to nearest even, the conversion instruction's rule).
+    static __device__ inline k8x8 quantize_q8(u32x4 u, float inv) {
+        const unsigned w[4] = {u[0], u[1], u[2], u[3]};
+        int lo = 0, hi = 0;
+        float x[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            x[2 * j] = __uint_as_float(w[j] << 16) * inv;               // below 256 in magnitude: no clamp needed
+            x[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u) * inv;
+        }
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], lo, false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(x[2], x[3], lo, true);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(x[4], x[5], hi, false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(x[6], x[7], hi, true);
+        return (k8x8)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
     }
 
     static __device__ inline Frag read_k(const char* stage, const Lane& L, int kb, int c) {
@@ -489,15 +523,18 @@ struct Prefill {
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
         const int qtok0 = it.tok_m;                        // token index of the block's first real token
         const unsigned smem_lds = lds_addr_of(smem);
-        const int sk_bytes = (int)p.k32_t * ESZ, sv_bytes = (int)p.v32_t * 2;
+        const int sk_bytes = F8 ? D : (int)p.k32_t * 2, sv_bytes = (int)p.v32_t * 2;
 
-        const char* kbase = reinterpret_cast<const char*>(p.k) + ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh) * ESZ;
+        // fp8: K comes from the quantised copy (token stride D bytes); Q is read as bf16 and converted in registers
+        const char* kbase = F8 ? reinterpret_cast<const char*>(p.k8) + ((unsigned long long)p.k8_b * (unsigned)b + (unsigned long long)p.k8_h * (unsigned)kvh)
+                               : reinterpret_cast<const char*>(p.k) + ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh) * 2;
         const char* vbase = reinterpret_cast<const char*>(p.v) + ((unsigned long long)p.v32_b * (unsigned)b + (unsigned long long)p.v32_h * (unsigned)kvh) * 2;
-        // fp8 Q/K: the two dequantisation scales of this (sequence, head) pair go into the softmax scale
+        // fp8: every query row is quantised in registers with its own scale (absmax of the row / 448: each lane owns
+        // one row, so the scale is a per-lane factor of the softmax scale); K carries one scale per (sequence, kv head)
         float sc2 = p.scale_log2;
         if constexpr (F8) {
             float f = 0.f;
-            if (lane == 0) f = p.qk_scales[(long long)b * p.Nq + head] * p.qk_scales[(long long)p.B * p.Nq + (long long)b * p.Nkv + kvh];
+            if (lane == 0) f = p.qk_scales[(long long)b * p.Nkv + kvh];
             sc2 *= __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, f)));
         }
 
@@ -526,24 +563,25 @@ struct Prefill {
         // early (they come from HBM; only the tile table's load, which the walk needs first, goes before them):
         // the rest of the set-up runs under their latency.
         Frag qf[D / 16];
+        u32x4 qraw[F8 ? D / 16 : 1];       // fp8: the bf16 rows as loaded, converted once they have arrived
         {
             const char* qrow = reinterpret_cast<const char*>(p.q) +
                                ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)head +
-                                (unsigned long long)p.q32_t * (unsigned)(qtok0 + row0)) * ESZ;
+                                (unsigned long long)p.q32_t * (unsigned)(qtok0 + row0)) * 2;
             // rows past the block's end load its last row instead (no per-lane branches around the loads):
             // what such rows compute is never stored
             const int last = len_m - 1 - row0;
-            const int qoff = ((ln < last ? ln : last) * (int)p.q32_t + lh * 8) * ESZ;
+            const int qoff = ((ln < last ? ln : last) * (int)p.q32_t + lh * 8) * 2;
             if (rb_active) {
 #pragma unroll
                 for (int c = 0; c < D / 16; ++c) {
-                    if constexpr (F8) qf[c] = *reinterpret_cast<const k8x8*>(qrow + qoff + c * 16);
+                    if constexpr (F8) qraw[c] = *reinterpret_cast<const u32x4*>(qrow + qoff + c * 32);
                     else qf[c] = as_bf16x8(ld16(qrow + qoff + c * 32));
                 }
             } else {
 #pragma unroll
                 for (int c = 0; c < D / 16; ++c) {
-                    if constexpr (F8) qf[c] = 0;
+                    if constexpr (F8) qraw[c] = u32x4{0u, 0u, 0u, 0u};
                     else qf[c] = as_bf16x8(uint4{0u, 0u, 0u, 0u});
                 }
             }
@@ -592,6 +630,23 @@ struct Prefill {
         // tell the compiler the Q fragments are in registers now: otherwise it would put its own
         // "wait for every outstanding load" in front of the first MFMA of each iteration, which would
         // also wait for the next tile's DMA and undo the overlap
+        if constexpr (F8) {
+            float amax = 0.f;
+#pragma unroll
+            for (int c = 0; c < D / 16; ++c) {
+                asm volatile("" : "+v"(qraw[c]));
+                const unsigned w[4] = {qraw[c][0], qraw[c][1], qraw[c][2], qraw[c][3]};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    amax = fmaxf(amax, fmaxf(fabsf(__uint_as_float(w[j] << 16)), fabsf(__uint_as_float(w[j] & 0xffff0000u))));
+            }
+            amax = fmaxf(amax, __shfl_xor(amax, 32));      // the other half of the row's dims
+            float q_scale, q_inv;
+            br_pow2_scale(amax, q_scale, q_inv);
+            sc2 *= q_scale;
+#pragma unroll
+            for (int c = 0; c < D / 16; ++c) qf[c] = quantize_q8(qraw[c], q_inv);
+        }
 #pragma unroll
         for (int c = 0; c < D / 16; ++c) asm volatile("" : "+v"(qf[c]));
         __syncthreads();
@@ -736,6 +791,7 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     __shared__ __attribute__((aligned(1024))) char smem[Smem<D, F8>::total(NW) + 2 * sizeof(BrDescMail)];
     BrDescMail* mail = reinterpret_cast<BrDescMail*>(smem + Smem<D, F8>::total(NW));
     using PF = Prefill<D, NW, F8>;
+    using PF16 = Prefill<D, NW, false>;
     const int NHG = p.geom.NHG;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
@@ -748,6 +804,20 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
         }
     }
     const typename PF::Lane L = PF::make_lane(p, wave, lane);
+    // fp8 kernel: the query block's items (the rows the document scores are read from, and the single block of a
+    // sequence without documents) run on the bf16 Q and K, every other item on the e4m3 copies
+    typename PF16::Lane L16;
+    if constexpr (F8) {
+        // only the K pieces differ between the two element types: the V offsets are shared registers
+        const typename PF16::Lane t = PF16::make_lane(p, wave, lane);
+#pragma unroll
+        for (int j = 0; j < PF16::JOK; ++j) L16.koff[j] = t.koff[j];
+        L16.krd = t.krd;
+#pragma unroll
+        for (int j = 0; j < PF16::JO; ++j) L16.voff[j] = L.voff[j];
+#pragma unroll
+        for (int d = 0; d < D / 32; ++d) L16.vrd[d] = L.vrd[d];
+    }
     // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
     for (int i = threadIdx.x * 16; i < Smem<D, F8>::total(NW); i += NW * 64 * 16) *reinterpret_cast<uint4*>(smem + i) = uint4{0u, 0u, 0u, 0u};
     const bool padded_layout = uni(hdr[BR_PH_PACKED]) == 0;
@@ -768,7 +838,12 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
         const int hg = BR_W(BR_ITEM_INTS);          // .hg
 #undef BR_W
         if (wave == 0) pf.draw();
-        PF::run_item(p, pv, it, hg, smem, L, pf, padded_layout);
+        if constexpr (F8) {
+            if (it.m == p.M - 1) PF16::run_item(p, pv, it, hg, smem, L16, pf, padded_layout);
+            else PF::run_item(p, pv, it, hg, smem, L, pf, padded_layout);
+        } else {
+            PF::run_item(p, pv, it, hg, smem, L, pf, padded_layout);
+        }
         if (wave == 0) pf.publish(&mail[cur ^ 1]);
         __syncthreads();
     }

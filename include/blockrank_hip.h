@@ -122,18 +122,23 @@ int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out
                           void* workspace, size_t workspace_bytes, int score_rows, float* score_part,
                           size_t score_part_bytes, void* stream, void* ev_start, void* ev_stop);
 
-/* Bytes of scratch br_prefill_fwd_fp8qk needs: the split-KV partials plus the quantised Q and K.
+/* Bytes of scratch br_prefill_fwd_fp8qk needs: the split-KV partials plus the quantised K and its scales.
  * tokens: length of the token axis summed over the batch (B*M*H for the padded layout, the number of
  * real tokens for a packed one). */
 size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int64_t tokens);
 
-/* br_prefill_fwd_scores with Q K^T computed in fp8 e4m3 and P V in bf16.  q, k, v, out are bf16 as in
- * br_prefill_fwd; Q and K are first quantised per (sequence, head) with scale = max|x| / 448 over the
- * real tokens (x / scale rounded to e4m3), the products run on the fp8 matrix cores and the two scales
- * are folded into the softmax scale.  D = 128 only.  score_part may be NULL (then score_rows is
- * ignored).  No reference counterpart: the reference computes Q K^T in the model dtype
- * (blockrank_std_attention.py:549-620); this is the reduced-precision variant for Qwen2.5-shaped
- * ranking whose scores must stay within 5e-3 relative of the fp32 result with the same top-10. */
+/* br_prefill_fwd_scores with the Q K^T products of the prefix and document blocks computed in fp8 e4m3
+ * and P V in bf16.  q, k, v, out are bf16 as in br_prefill_fwd.  K is first quantised per (sequence, kv
+ * head) with the power-of-two scale 2^(floor(log2(max|x|)) - 7), the maximum taken over the real tokens
+ * (x / scale rounded to e4m3, written into the workspace); Q is converted by the attention kernel itself,
+ * in registers, every query row with the scale its own maximum gives by the same rule (a power of two
+ * makes the division exact); the products run on the fp8 matrix cores and the scales are folded into the
+ * softmax scale.  The query block's rows - the ones the per-document scores are read from - are computed
+ * on the bf16 Q and K, so the score partials are those of br_prefill_fwd_scores.  D = 128 only.
+ * score_part may be NULL (then score_rows is ignored).  No reference counterpart: the reference computes
+ * Q K^T in the model dtype (blockrank_std_attention.py:549-620); this is the reduced-precision variant
+ * for Qwen2.5-shaped ranking whose scores must stay within 5e-3 relative of the fp32 result with the
+ * same top-10. */
 int br_prefill_fwd_fp8qk(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
                          int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
                          const int64_t* v_strides, const int64_t* out_strides, float scale, int64_t tokens,

@@ -400,21 +400,30 @@ def eval_labels(valid: np.ndarray) -> np.ndarray:
     return labels
 
 
-def quantize_fp8_e4m3(x: torch.Tensor, valid: torch.Tensor) -> torch.Tensor:
-    """Per-(sequence, head) absmax quantisation to fp8 e4m3 and back, as the fp8 Q K^T variant defines
-    it (no reference counterpart; the Qwen2.5-7B-shaped benchmark configuration): scale = max |x| over the sequence's real tokens
-    / 448; x / scale rounded to the nearest e4m3 value (torch.float8_e4m3fn, round to nearest even,
-    the same format the gfx950 conversion instruction produces); returned dequantised, in float32.
-    x (B, heads, S, D); valid (B, M, H) with M*H = S.  Pinned by: values that are exactly representable
-    survive unchanged; the round trip error is at most 2^-4 relative for normal values; the largest
-    magnitude of every (sequence, head) is reproduced exactly."""
+def quantize_fp8_e4m3(x: torch.Tensor, valid: torch.Tensor, per_row: bool = False) -> torch.Tensor:
+    """Quantisation to fp8 e4m3 and back, as the fp8 Q K^T variant defines it (no reference counterpart; the
+    Qwen2.5-7B-shaped benchmark configuration).  One power-of-two scale per group, 2^(floor(log2(max |x|)) - 7),
+    which puts the group's largest magnitude into [128, 256) of e4m3's range (largest value 448); the group is the
+    sequence's real tokens of one head (per_row=False: how K is quantised) or one token of one head
+    (per_row=True: how the query rows are).  x / scale is rounded to the nearest e4m3 value (torch.float8_e4m3fn,
+    round to nearest even, the same format the gfx950 conversion instruction produces) and returned dequantised,
+    in float32.  A power-of-two scale makes the division exact: 16-bit inputs land on exact ties of the e4m3 grid
+    often (one element in a thousand), and an inexact scale would break them differently from one implementation
+    to the next.  A group whose maximum is below 2^-119 counts as zero.
+    x (B, heads, S, D); valid (B, M, H) with M*H = S.  Pinned by: values with at most four significant bits
+    within 2^9 of the group's maximum survive unchanged; the round trip error is at most 2^-4 relative for normal
+    values; multiplying a group by a power of two multiplies its result by the same."""
     B, Hh, S, D = x.shape
     keep = valid.reshape(B, 1, S, 1).to(x.device)
     xf = x.float()
-    amax = torch.where(keep, xf.abs(), torch.zeros((), dtype=torch.float32)).amax(dim=(2, 3), keepdim=True)
-    scale = amax / 448.0
-    safe = torch.where(scale > 0, scale, torch.ones_like(scale))
-    q = (xf / safe).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).float()
+    amax = torch.where(keep, xf.abs(), torch.zeros((), dtype=torch.float32)).amax(dim=(3,) if per_row else (2, 3), keepdim=True)
+    amax = amax.clamp(max=3.0e38).contiguous()
+    ebits = amax.view(torch.int32) & 0x7F800000
+    ok = ebits >= (8 << 23)
+    sbits = torch.where(ok, ebits - (7 << 23), torch.full_like(ebits, 127 << 23))
+    scale = torch.where(ok, sbits.view(torch.float32), torch.zeros_like(amax))
+    inv = torch.where(ok, ((254 << 23) - sbits).view(torch.float32), torch.zeros_like(amax))
+    q = (xf * inv).to(torch.float8_e4m3fn).float()
     return torch.where(keep, q * scale, torch.zeros((), dtype=torch.float32))
 
 

@@ -102,26 +102,38 @@ def test_topk_is_stable_descending():
 
 
 def test_fp8_quantiser_pins():
-    """quantize_fp8_e4m3: representable values survive, the per-head maximum is exact, the relative
-    round-trip error of normal values is at most 2^-4, padded positions come back as zero."""
+    """quantize_fp8_e4m3: values with at most four significant bits survive, the relative round-trip error of
+    normal values is at most 2^-4, a power-of-two factor passes through, padded positions come back as zero."""
     import torch
     from oracle import blockrank_oracle as orc
     valid = torch.ones(1, 2, 4, dtype=torch.bool)
     valid[0, 0, 0] = False
-    # e4m3 values (scaled so that the maximum maps to 448): 448, 416, 1.0, 0.875, 2^-6 (smallest normal), 0
-    vals = torch.tensor([0.0, 448.0, -416.0, 1.0, 0.875, 2.0 ** -6, 3.5, -240.0])
+    # four significant bits, the largest (240) sets the scale 2^0; 2^-6 is e4m3's smallest normal value
+    vals = torch.tensor([0.0, 240.0, -208.0, 1.0, 0.875, 2.0 ** -6, 3.5, -120.0])
+    for factor in (1.0, 2.0 ** -11, 2.0 ** 5):        # any power-of-two factor must cancel
+        x = torch.zeros(1, 1, 8, 4)
+        x[0, 0, :, 0] = vals * factor
+        x[0, 0, 0, :] = 1e6                           # padded position: must not set the scale
+        got = orc.quantize_fp8_e4m3(x, valid)
+        assert torch.equal(got[0, 0, 0], torch.zeros(4))
+        assert torch.equal(got[0, 0, 1:, 0], x[0, 0, 1:, 0])
+    # five significant bits are rounded to four, ties to even: 17 -> 16, 19 -> 20, 18.5 -> 18
     x = torch.zeros(1, 1, 8, 4)
-    x[0, 0, :, 0] = vals * 0.37                       # any common factor must cancel
-    x[0, 0, 0, :] = 1e6                               # padded position: must not set the scale
+    x[0, 0, 1:5, 0] = torch.tensor([128.0, 17.0, 19.0, 18.5])
     got = orc.quantize_fp8_e4m3(x, valid)
-    assert torch.equal(got[0, 0, 0], torch.zeros(4))
-    torch.testing.assert_close(got[0, 0, 1:, 0], x[0, 0, 1:, 0], rtol=1e-6, atol=0)
+    assert got[0, 0, 1:5, 0].tolist() == [128.0, 16.0, 20.0, 18.0]
     g = torch.Generator().manual_seed(0)
     y = torch.randn(2, 3, 8, 16, generator=g)
     v2 = torch.ones(2, 2, 4, dtype=torch.bool)
-    r = orc.quantize_fp8_e4m3(y, v2)
-    amax = y.abs().amax(dim=(2, 3))
-    torch.testing.assert_close(r.abs().amax(dim=(2, 3)), amax, rtol=1e-6, atol=0)
-    normal = y.abs() >= (amax / 448.0 * 2.0 ** -6)[:, :, None, None]
-    rel = ((r - y).abs() / y.abs())[normal]
-    assert rel.max().item() <= 2.0 ** -4 + 1e-6
+    for per_row in (False, True):
+        r = orc.quantize_fp8_e4m3(y, v2, per_row=per_row)
+        amax = y.abs().amax(dim=(3,) if per_row else (2, 3), keepdim=True)
+        normal = y.abs() >= amax * 2.0 ** -13          # max / 2^7 >= 1 = 2^6 times the smallest normal value
+        rel = ((r - y).abs() / y.abs())[normal.expand_as(y)]
+        assert rel.max().item() <= 2.0 ** -4 + 1e-6
+        assert torch.equal(orc.quantize_fp8_e4m3(y * 2.0 ** -9, v2, per_row=per_row) * 2.0 ** 9, r)
+    # one scale per row: a row of tiny values keeps its relative precision
+    tiny = y.clone()
+    tiny[:, :, 3] *= 2.0 ** -14
+    rt = orc.quantize_fp8_e4m3(tiny, v2, per_row=True)
+    assert torch.equal(rt[:, :, 3] * 2.0 ** 14, orc.quantize_fp8_e4m3(y, v2, per_row=True)[:, :, 3])
