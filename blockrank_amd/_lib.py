@@ -33,6 +33,9 @@ SIGNATURES = {
     "br_prefill_workspace_bytes_fused": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "br_prefill_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t, c_void_p]),
+    "br_prefill_noalloc_max_workspace_bytes": (c_size_t, []),
+    "br_prefill_fwd_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                       c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "br_prefill_fwd_events": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t, c_void_p,
                                       c_void_p, c_void_p]),

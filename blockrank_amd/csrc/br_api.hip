@@ -1,5 +1,6 @@
 // extern "C" entry points of libblockrank_hip.so: argument checks, geometry selection, launches.
 #include <stdarg.h>
+#include <atomic>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -32,6 +33,12 @@ int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, hipStream_t str
 int br_launch_rmsnorm(const void* x, const void* w, void* out, long long rows, int hidden, long long sx, long long so, float eps, int dtype,
                       int n_cu, hipStream_t stream);
 void br_launch_silu_mul(const void* gate, const void* up, void* out, long long n, int dtype, int n_cu, hipStream_t stream);
+
+// Split-KV partials of br_prefill_fwd_noalloc: device memory that belongs to the library, one copy on every GPU
+// the library runs on, held until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress: the address the kernels get is the one that call returns for the current device.
+#define BR_NOALLOC_SCRATCH_BYTES ((size_t)80 << 20)
+static __device__ __align__(256) unsigned char scratch[BR_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -316,6 +323,42 @@ int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const
                    const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
                         workspace, workspace_bytes, stream, nullptr, nullptr, 0, nullptr, 0);
+}
+
+size_t br_prefill_noalloc_max_workspace_bytes(void) { return BR_NOALLOC_SCRATCH_BYTES; }
+
+// Address of this device's copy of the scratch array, looked up once per device (with that device current).
+static int noalloc_scratch(void** out) {
+    constexpr int kMaxDev = 64;
+    static std::atomic<void*> ptrs[kMaxDev];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(BR_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDev) return fail(BR_ERR_HIP, "device index %d out of range", dev);
+    void* ptr = ptrs[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) return fail(BR_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        ptrs[dev].store(ptr, std::memory_order_release);     // every thread gets the same address for a device
+    }
+    *out = ptr;
+    return BR_OK;
+}
+
+int br_prefill_fwd_noalloc(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                           int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                           const int64_t* out_strides, float scale, int dtype, void* stream) {
+    int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
+    if (rc) return rc;
+    const size_t need = br_prefill_workspace_bytes(B, Nq, Nkv, D);
+    if (need > BR_NOALLOC_SCRATCH_BYTES)
+        return fail(BR_ERR_SPACE, "br_prefill_fwd_noalloc: B=%d with %d/%d heads of dim %d needs %zu bytes of partials, the built-in scratch holds %zu; "
+                                  "use br_prefill_fwd with a workspace, or a smaller batch", B, Nq, Nkv, D, need, (size_t)BR_NOALLOC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if ((rc = noalloc_scratch(&ws))) return rc;
+    // exactly `need` bytes are offered, so the call can never take the path that wants the larger (fused) workspace
+    return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
+                        ws, need, stream, nullptr, nullptr, 0, nullptr, 0);
 }
 
 int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,

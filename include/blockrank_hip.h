@@ -105,6 +105,20 @@ int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out
                           const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype,
                           void* workspace, size_t workspace_bytes, void* stream, void* ev_start, void* ev_stop);
 
+/* br_prefill_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * result as br_prefill_fwd without the workspace: the split-KV partials live in a device array that
+ * belongs to the library (br_prefill_noalloc_max_workspace_bytes() = 80 MiB on every GPU the library is
+ * used on, until the process ends).  Neither this call nor anything it calls allocates or frees memory.
+ * A request whose br_prefill_workspace_bytes() exceeds that size is refused with BR_ERR_SPACE (Mistral-7B
+ * heads: B <= 4).  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream, one after the other, do not.  Nothing in the array has
+ * to be cleared between calls (a call reads only the partials it wrote itself). */
+size_t br_prefill_noalloc_max_workspace_bytes(void);
+int br_prefill_fwd_noalloc(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
+                           int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
+                           const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype, void* stream);
+
 /* Bytes of the score-partials buffer of br_prefill_fwd_scores. */
 size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows);
 

@@ -54,6 +54,10 @@ def test_pure_host_entry_points():
     rc = lib.br_prefill_bwd(None, None, None, None, None, None, None, 1, 4, 2, 3, 8, 96, None, None, None, None, None, None,
                             None, None, None, None, None, None, 1.0, 24, None, 0, None)
     assert rc == _lib.BR_ERR_ARG and b"head dim" in lib.br_last_error()
+    # the entry point that allocates nothing refuses a request beyond its built-in scratch, before any device call
+    assert lib.br_prefill_noalloc_max_workspace_bytes() == 80 << 20
+    rc = lib.br_prefill_fwd_noalloc(None, None, None, None, None, 5, 32, 8, 22, 160, 128, None, None, None, None, 1.0, 1, None)
+    assert rc == _lib.BR_ERR_SPACE and b"built-in scratch" in lib.br_last_error()
     # argument errors come back as codes with a message, before anything touches a device
     rc = lib.br_prefill_fwd(None, None, None, None, None, 1, 4, 2, 3, 8, 96, None, None, None, None, 1.0, 1, None, 0, None)
     assert rc == _lib.BR_ERR_ARG and b"head dim" in lib.br_last_error()
