@@ -19,10 +19,39 @@ from .attention import _DTYPE_CODE, _dense_last_dim, _stream_ptr
 _I64x2 = _lib.ctypes.c_int64 * 2
 
 
+class _RotaryWithGrad(torch.autograd.Function):
+    """The rotation with its backward.  With x = (x1, x2) the two halves of the head dim, y1 = x1 c1 - x2 s1 and
+    y2 = x2 c2 + x1 s2, so dx1 = g1 c1 + g2 s2 and dx2 = g2 c2 - g1 s1: the same kernel applied to the incoming
+    gradient with the sine table's halves exchanged and negated (no assumption that the two halves of cos / sin
+    are equal).  cos and sin are position tables, not parameters: they get no gradient."""
+
+    @staticmethod
+    def forward(ctx, q, k, cos, sin):
+        ctx.save_for_backward(cos, sin)
+        return _rotate(q, k, cos, sin)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, gq, gk):
+        cos, sin = ctx.saved_tensors
+        sin_t = -torch.roll(sin, sin.shape[-1] // 2, dims=-1)
+        dq, dk = _rotate(gq, gk, cos, sin_t)
+        return dq, dk, None, None
+
+
 def apply_rotary_pos_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqueeze_dim: int = 1):
     """q (B, Nq, S, D), k (B, Nkv, S, D) (any strides with a dense last dim, e.g. the head-transposed views of
     the projections), cos / sin (B or 1, S, D).  Returns (q_embed, k_embed) with the same logical shapes, stored
-    as (B, S, heads, D) - what the attention hook takes without a copy.  bf16 or fp32, D 64 or 128, CUDA tensors."""
+    as (B, S, heads, D) - what the attention hook takes without a copy.  bf16 or fp32, D 64 or 128, CUDA tensors.
+    Differentiable with respect to q and k (the backward is the same kernel on the gradients)."""
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad):
+        if cos.requires_grad or sin.requires_grad:
+            raise NotImplementedError("gradients with respect to the cos / sin tables are not implemented")
+        return _RotaryWithGrad.apply(q, k, cos, sin)
+    return _rotate(q, k, cos, sin, unsqueeze_dim)
+
+
+def _rotate(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqueeze_dim: int = 1):
     assert unsqueeze_dim == 1, "only the (batch, heads, tokens, dim) convention of the decoder layers is supported"
     assert q.is_cuda and k.is_cuda and cos.is_cuda and sin.is_cuda, "the rotary embedding kernel needs device tensors"
     assert q.dtype == k.dtype == cos.dtype == sin.dtype and q.dtype in _DTYPE_CODE, "q, k, cos and sin must share a dtype (bf16 or fp32)"

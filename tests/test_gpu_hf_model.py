@@ -166,3 +166,89 @@ def test_training_step_gradients_match_eager_autograd():
         rel16 = ((eager16[n] - w).norm() / w.norm()).item()
         cos = torch.nn.functional.cosine_similarity(ours[n].flatten(), w.flatten(), dim=0).item()
         assert rel <= max(1.5 * rel16, 2e-2) and cos >= 0.99, f"{n}: relative gradient error {rel:.3e} (eager bf16: {rel16:.3e}), cosine {cos:.5f}"
+
+
+def _eager_scores(mdl, dtype, lay, ids, pos, layer_idx, bracket_from_end=1):
+    """Per-document scores of scripts/eval_attn.py:139-151 from the library's own eager attention: the model under the
+    dense additive mask of the oracle's predicate, the scoring layer's probabilities on rows {bracket - 1, bracket},
+    renormalised over the document columns (a softmax restricted to them, losses.py:56-59), summed per document,
+    mean over heads and the two rows, divided by the temperature (losses.py:64-74)."""
+    B, S, M, H = lay.B, lay.S, lay.M, lay.H
+    ok = torch.as_tensor(orc.allowed(lay.valid.numpy())) | torch.eye(S, dtype=torch.bool)[None]
+    add = torch.zeros(B, 1, S, S, dtype=dtype).masked_fill_(~ok[:, None], torch.finfo(dtype).min).to(DEV)
+    mdl.set_attn_implementation("eager")
+    with torch.no_grad():
+        ref = mdl(input_ids=ids, position_ids=pos, attention_mask=add, output_attentions=True, use_cache=False)
+    br_row = S - 1 - bracket_from_end
+    p = ref.attentions[layer_idx][:, :, br_row - 1:br_row + 1, H:S - H].double()
+    p = p / p.sum(dim=-1, keepdim=True)
+    return (p.reshape(B, p.shape[1], 2, M - 2, H).sum(-1).mean(dim=(1, 2)) / 0.05).cpu()
+
+
+def _ranker_inputs(lay, vocab, seed):
+    lay.labels[:] = -100
+    lay.labels[:, -2:] = 7                                   # "[" is the second to last token
+    ids = torch.randint(0, vocab, (lay.B, lay.S), generator=torch.Generator().manual_seed(seed)).to(DEV)
+    return ids, lay.position_ids.to(DEV), lay.valid.to(DEV), lay.labels.to(DEV)
+
+
+def _packed_call(ranker, lay, ids, pos):
+    keep = lay.valid.reshape(-1).to(DEV)
+    lens = torch.as_tensor(lay.lengths, dtype=torch.int32, device=DEV)
+    h1 = min(16, lay.H)
+    rows = torch.tensor([[h1 - 3, h1 - 2]] * lay.B, dtype=torch.int32, device=DEV)       # bracket = second to last token
+    return ranker.forward_packed(ids.reshape(-1)[keep][None], pos.reshape(-1)[keep][None], lens, rows, H=lay.H)
+
+
+@pytest.mark.parametrize("kind", ["mistral", "qwen2"])
+def test_truncated_ranker_against_eager_model_under_the_oracle_mask(kind):
+    """The layer-truncated driver, padded and packed entry, against scores computed without any of this package's
+    kernels: fp32 weights, so the comparison is tight (1e-3 relative, same order)."""
+    import copy
+    br.register_triton_blockrank_attention()
+    model = build(kind, torch.float32)
+    lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
+    ids, pos, valid, labels = _ranker_inputs(lay, 512, 3)
+    for layer_idx in (1, 2):
+        want = _eager_scores(model, torch.float32, lay, ids, pos, layer_idx).numpy()
+        model.set_attn_implementation("triton_blockrank")
+        ranker = br.TruncatedRanker(model, layer_idx)
+        got = ranker(ids, valid, pos, labels=labels)
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-3)
+        got_p = _packed_call(ranker, lay, ids, pos)
+        np.testing.assert_allclose(got_p.cpu().numpy(), want, rtol=1e-3)
+        assert (orc.topk_indices(got.cpu().numpy(), 3) == orc.topk_indices(want, 3)).all()
+    # bf16 weights (what ranking runs in): as close to the fp32 result as the eager bf16 model is
+    m16 = copy.deepcopy(model).to(torch.bfloat16)
+    e16 = _eager_scores(m16, torch.bfloat16, lay, ids, pos, 2).numpy()
+    m16.set_attn_implementation("triton_blockrank")
+    r16 = br.TruncatedRanker(m16, 2)
+    yard = np.abs(e16 - want).max()
+    for got in (r16(ids, valid, pos, labels=labels), _packed_call(r16, lay, ids, pos)):
+        assert np.abs(got.cpu().numpy() - want).max() <= max(1.5 * yard, 1e-3 * np.abs(want).max())
+
+
+def test_truncated_ranker_at_7b_width():
+    """Mistral-7B layer shapes (hidden 4096, 32 / 8 heads of 128, MLP 14336), three layers, one ranking request of the
+    end-to-end benchmark configuration (64-token prefix, 20 documents U[96, 224], 32-token query), bf16 through the
+    truncated driver against the fp32 eager model under the oracle's mask; the yardstick is the eager model in bf16."""
+    import copy
+    from transformers import MistralConfig, MistralForCausalLM
+    br.register_triton_blockrank_attention()
+    torch.manual_seed(0)
+    cfg = MistralConfig(vocab_size=2048, hidden_size=4096, intermediate_size=14336, num_hidden_layers=3, num_attention_heads=32,
+                        num_key_value_heads=8, head_dim=128, max_position_embeddings=32768, rope_theta=1e6, sliding_window=None)
+    model = MistralForCausalLM(cfg).to(DEV, torch.bfloat16).eval()
+    lay = synthetic.random_layout(1, 64, 20, 96, 224, 32, seed=0)
+    ids, pos, valid, labels = _ranker_inputs(lay, 2048, 4)
+    want = _eager_scores(copy.deepcopy(model).float(), torch.float32, lay, ids, pos, 2).numpy()
+    e16 = _eager_scores(model, torch.bfloat16, lay, ids, pos, 2).numpy()
+    model.set_attn_implementation("triton_blockrank")
+    ranker = br.TruncatedRanker(model, 2)
+    yard = np.abs(e16 - want).max()
+    assert yard <= 0.05 * np.abs(want).max(), "the bf16 eager model itself should be within a few percent"
+    for got in (ranker(ids, valid, pos, labels=labels), _packed_call(ranker, lay, ids, pos)):
+        g = got.cpu().numpy()
+        assert g.shape == (1, 20)
+        assert np.abs(g - want).max() <= max(1.5 * yard, 1e-3 * np.abs(want).max()), (np.abs(g - want).max(), yard)
+        np.testing.assert_allclose(g.sum(-1) * 0.05, 1.0, rtol=1e-3)

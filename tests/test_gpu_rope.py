@@ -91,3 +91,58 @@ def test_patched_model_and_ranker_agree_with_unpatched(kind):
     import sys
     mod = sys.modules[type(model.model.layers[0].self_attn).__module__]
     assert mod.apply_rotary_pos_emb.__module__ != "blockrank_amd.rope", "unpatch_rotary must restore the model's own function"
+
+
+def test_gradients_match_the_eager_expression():
+    """The rotation is differentiable in q and k: its backward (the same kernel on the gradients) against autograd
+    through the model file's expression in float64, with tables whose two halves differ."""
+    B, Nq, Nkv, S, D = 2, 4, 2, 19, 64
+    g = torch.Generator().manual_seed(3)
+    q, k, _, _ = _inputs(B, Nq, Nkv, S, D, torch.float32, seed=7)
+    ang = torch.rand(B, S, D, generator=g) * 6.28                       # halves not equal
+    cos, sin = ang.cos().to(DEV), (ang * 1.3).sin().to(DEV)
+    wq, wk = torch.randn(q.shape, generator=g).to(DEV), torch.randn(k.shape, generator=g).to(DEV)
+    q1, k1 = q.clone().requires_grad_(), k.clone().requires_grad_()
+    qo, ko = br.apply_rotary_pos_emb(q1, k1, cos, sin)
+    assert qo.requires_grad and ko.requires_grad
+    ((qo * wq).sum() + (ko * wk).sum()).backward()
+    q2, k2 = q.double().requires_grad_(), k.double().requires_grad_()
+    eq, ek = _eager(q2, k2, cos.double(), sin.double())
+    ((eq * wq.double()).sum() + (ek * wk.double()).sum()).backward()
+    assert (q1.grad.double() - q2.grad).abs().max().item() <= 1e-5
+    assert (k1.grad.double() - k2.grad).abs().max().item() <= 1e-5
+
+
+def test_patched_model_trains_through_the_rotation():
+    """After patch_rotary the projections in front of the rotation still get their gradients: q_proj / k_proj of a
+    small Mistral, patched against unpatched, same loss."""
+    from tests.test_gpu_hf_model import build
+    br.register_blockrank_attention()
+    model = build("mistral", torch.float32)
+    model.set_attn_implementation("default_blockrank")
+    lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
+    ids = torch.randint(0, 512, (lay.B, lay.S), generator=torch.Generator().manual_seed(1)).to(DEV)
+    pos, valid = lay.position_ids.to(DEV), lay.valid.to(DEV)
+    rows = lay.valid.reshape(lay.B, lay.S).to(DEV)
+    probe = torch.randn((lay.B, lay.S, 256), generator=torch.Generator().manual_seed(2)).to(DEV)
+
+    def step():
+        model.zero_grad()
+        # fp32 inputs have no attention backward here: the eager library attention under a dense mask carries the graph
+        ok = torch.as_tensor(orc.allowed(lay.valid.numpy())) | torch.eye(lay.S, dtype=torch.bool)[None]
+        add = torch.zeros(lay.B, 1, lay.S, lay.S).masked_fill_(~ok[:, None], torch.finfo(torch.float32).min).to(DEV)
+        model.set_attn_implementation("eager")
+        out = model(input_ids=ids, position_ids=pos, attention_mask=add, output_hidden_states=True, use_cache=False)
+        (out.hidden_states[-1] * probe)[rows].sum().backward()
+        return {n: p.grad.clone() for n, p in model.named_parameters() if "q_proj" in n or "k_proj" in n}
+
+    ref = step()
+    br.patch_rotary(model)
+    try:
+        got = step()
+    finally:
+        br.unpatch_rotary(model)
+    assert ref.keys() == got.keys() and len(ref) == 6
+    for n in ref:
+        assert got[n].abs().max().item() > 0
+        torch.testing.assert_close(got[n], ref[n], rtol=1e-3, atol=1e-5 * ref[n].abs().max().item() + 1e-7)
