@@ -541,14 +541,25 @@ def last_block_logits(query, key, block_mask, rows, scaling: float, neg: Optiona
         neg = 0.7 * torch.finfo(query.dtype).min
     lib = _lib.load()
     dev = query.device
+    MH = bm.M * bm.H
     with torch.cuda.device(dev):
         plan = bm.plan(Nq, Nkv)
         # (for a packed layout too the result is laid out over the M*H padded key slots, like the reference's)
-        out = torch.empty((B, Nq, R, bm.M * bm.H), dtype=torch.float32, device=dev)
-        _lib.check(lib.br_last_block_logits(
-            q.data_ptr(), k.data_ptr(), plan.data_ptr(), rows.data_ptr(), R, B, Nq, Nkv, bm.M, bm.H, D,
-            _lib.strides3(q, bm.packed), _lib.strides3(k, bm.packed), float(scaling), float(neg), _DTYPE_CODE[query.dtype],
-            out.data_ptr(), _stream_ptr(dev)))
+        if R <= 16:
+            out = torch.empty((B, Nq, R, MH), dtype=torch.float32, device=dev)
+            chunks = [(rows, out)]
+        else:
+            # the kernel takes up to 16 rows per call (the reference's default num_last_queries); more rows go in
+            # groups of 16, each into its own buffer, joined at the end
+            chunks = [(rows[:, r0:r0 + 16].contiguous(), torch.empty((B, Nq, min(16, R - r0), MH), dtype=torch.float32, device=dev))
+                      for r0 in range(0, R, 16)]
+        for rws, dst in chunks:
+            _lib.check(lib.br_last_block_logits(
+                q.data_ptr(), k.data_ptr(), plan.data_ptr(), rws.data_ptr(), rws.shape[1], B, Nq, Nkv, bm.M, bm.H, D,
+                _lib.strides3(q, bm.packed), _lib.strides3(k, bm.packed), float(scaling), float(neg), _DTYPE_CODE[query.dtype],
+                dst.data_ptr(), _stream_ptr(dev)))
+        if R > 16:
+            out = torch.cat([d for _, d in chunks], dim=2)
     return out
 
 
@@ -616,7 +627,10 @@ def blockrank_attention_forward(
     if groups is not None:
         assert key.shape[1] * groups == Nq, "num_key_value_groups does not match the query/key head counts"
     if dropout > 0.0 and getattr(module, "training", False):
-        warnings.warn("Dropout is not supported in kernelized BlockRank attention, ignoring dropout parameter")
+        # the reference's trainable hooks apply attention dropout in training (blockrank_std_attention.py:168-169, :551);
+        # its kernelised hook ignores it with a warning (blockrank_triton_kernel_attention.py:844-846).  Ignoring it
+        # silently changes what is trained, so refuse.
+        raise NotImplementedError("attention dropout > 0 in training is not supported by the HIP attention (set attention_dropout=0)")
 
     layers = kwargs.get("layers_to_return_scores", None)
     if layers is not None:

@@ -90,7 +90,9 @@ def block_icr_collate_packed(batch: List[dict], pad_to_multiple_of: Optional[int
         # the completion starts at position last_prompt of the last block; in a block of H slots
         # whose tokens sit at the end that is slot H - n + last_prompt, i.e. this index into the last h1
         bracket = h1 - int(kept[-1]) + min(last_prompt, int(kept[-1]))
-        assert bracket >= 1, "Bracket token not found in last h1 positions."
+        # (a completion that truncation removed altogether has no bracket row: the reference fails the same way,
+        # losses.py:46-48)
+        assert 1 <= bracket <= h1 - 1 and last_prompt < int(kept[-1]), "Bracket token not found in last h1 positions."
         rows.append([bracket - 1, bracket])
     out = {
         "input_ids": torch.cat(ids)[None],

@@ -57,10 +57,8 @@ int fail(int code, const char* fmt, ...) {
 bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW) {
     if (Nq <= 0 || Nkv <= 0 || Nq % Nkv) return false;
     const int G = Nq / Nkv;
-    // experiment knob: BLOCKRANK_MAX_GW caps the heads one workgroup covers
-    static const int max_gw = getenv("BLOCKRANK_MAX_GW") ? atoi(getenv("BLOCKRANK_MAX_GW")) : 8;
     int Gw = 1;
-    for (int d = 1; d <= 8 && d <= G && d <= max_gw; ++d)
+    for (int d = 1; d <= 8 && d <= G; ++d)
         if (G % d == 0) Gw = d;
     int nw, tpb;
     switch (Gw) {
@@ -69,12 +67,6 @@ bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW) {
         case 3: nw = 6; tpb = 2; break;
         case 4: nw = 4; tpb = 1; break;
         default: nw = Gw; tpb = 1; break;
-    }
-    // experiment knob: BLOCKRANK_WIDE_TILES=1 doubles the tokens per tile where 8 waves allow it
-    static const bool wide = getenv("BLOCKRANK_WIDE_TILES") && atoi(getenv("BLOCKRANK_WIDE_TILES")) != 0;
-    if (wide && nw == 4) {
-        nw = 8;
-        tpb *= 2;
     }
     g->G = G;
     g->Gw = Gw;
@@ -248,8 +240,8 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     // computed with each block) needs M-dependent room for partials.  It is opt-in for now - with
     // BLOCKRANK_AMD_RESIDENT=1, and only when the caller's workspace has that room: on the measured
     // workloads it does not beat the streaming kernel yet.
-    const char* res_env = getenv("BLOCKRANK_AMD_RESIDENT");
-    const bool fused = dtype == BR_DTYPE_BF16 && fp8_tokens == 0 && !lse && (D == 64 || D == 128) && res_env && atoi(res_env) != 0 &&
+    static const bool res_env = getenv("BLOCKRANK_AMD_RESIDENT") && atoi(getenv("BLOCKRANK_AMD_RESIDENT")) != 0;   // read once per process
+    const bool fused = dtype == BR_DTYPE_BF16 && fp8_tokens == 0 && !lse && (D == 64 || D == 128) && res_env &&
                        workspace_bytes >= br_prefill_workspace_bytes_fused(B, M, Nq, Nkv, D);
     p.queue_view = fused ? 1 : 0;
     p.slots = fused ? br_slots_view1(M) : BR_SLOTS_PER_SEQ;

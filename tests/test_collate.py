@@ -61,3 +61,17 @@ def test_packed_collate_matches_padded_rules():
             assert torch.equal(got[key].long(), want[key].long()), key
         assert got["answer_ids"].shape == (len(items), 2)
         assert got["input_ids"].shape[1] == int(got["block_lengths"].sum())
+
+
+def test_completion_removed_by_truncation_is_refused():
+    """A last block so long that truncation to H cuts the completion off has no bracket token left: the reference's
+    score routine fails on such a batch (losses.py:46-48), and so does the packed collate function."""
+    import pytest
+    items = _items(seed=3, B=2, M=4)
+    long = dict(items[0])
+    lens = long["block_lengths"].clone()
+    lens[-2] = 40                                    # last prompt block alone reaches the cap
+    long["block_lengths"] = lens
+    long["input_ids"] = torch.randint(5, 500, (int(lens.sum()),))
+    with pytest.raises(AssertionError, match="Bracket token not found"):
+        block_icr_collate_packed([long, dict(items[1])], max_block_length=32)

@@ -128,3 +128,48 @@ def test_loss_api_handle_and_tensor_paths_agree():
     loss, acc, lg = br.compute_auxiliary_attention_loss(h, labels, lay.valid.to(DEV), answer_ids=torch.tensor([[0, -1], [2, 3]], device=DEV),
                                                         return_logits=True)
     assert torch.isfinite(loss) and 0 <= acc.item() <= 1 and torch.equal(lg, fused)
+
+
+def test_more_than_sixteen_score_rows_materialised():
+    """num_last_queries above 16 (the reference accepts any value, blockrank_std_attention.py:637-645): the dense
+    logits tensor is assembled from groups of 16 rows and equals the closed form row by row."""
+    lay = synthetic.uniform_layout(1, 16, 3, 48, 40)
+    Nq, Nkv, D = 4, 2, 64
+    q, k, v = synthetic.random_qkv(lay, Nq, Nkv, D, torch.float32, DEV, seed=8)
+
+    class Mod:
+        layer_idx = 0
+        num_key_value_groups = 2
+        training = False
+
+    mask = br.blockrank_attention_mask(batch_size=1, attention_mask=lay.valid.to(DEV), dtype=torch.float32)
+    _, t = br.blockrank_attention_forward(Mod(), q, k, v, mask, D ** -0.5, return_last_block_attn_scores=True, num_last_queries=37,
+                                          materialize_scores=True)
+    assert t.shape == (1, Nq, 37, lay.S)
+    _, t16 = br.blockrank_attention_forward(Mod(), q, k, v, mask, D ** -0.5, return_last_block_attn_scores=True, materialize_scores=True)
+    assert torch.equal(t[:, :, -16:], t16)
+    qq = q[:, :, -37:].double().cpu()
+    kk = k.double().cpu().repeat_interleave(2, dim=1)
+    want = torch.einsum("bnrd,bnsd->bnrs", qq, kk) * D ** -0.5
+    vis = lay.valid.reshape(1, 1, 1, lay.S).expand_as(want).clone()
+    for r in range(37):                              # causal inside the query block
+        vis[..., r, lay.S - 37 + r + 1:] = False
+    torch.testing.assert_close(t.double().cpu()[vis], want[vis], rtol=1e-5, atol=1e-5)
+    assert (t.cpu()[~vis] < -1e30).all()
+
+
+def test_dropout_in_training_is_refused():
+    lay = synthetic.uniform_layout(1, 16, 2, 32, 16)
+    q, k, v = synthetic.random_qkv(lay, 4, 2, 64, torch.bfloat16, DEV, seed=9)
+
+    class Mod:
+        layer_idx = 0
+        num_key_value_groups = 2
+        training = True
+
+    mask = br.blockrank_attention_mask(batch_size=1, attention_mask=lay.valid.to(DEV), dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="dropout"):
+        br.blockrank_attention_forward(Mod(), q, k, v, mask, 0.125, dropout=0.1)
+    Mod.training = False
+    out, _ = br.blockrank_attention_forward(Mod(), q, k, v, mask, 0.125, dropout=0.1)      # evaluation: dropout is off anyway
+    assert out.shape == (1, lay.S, 4, 64)
