@@ -30,7 +30,6 @@ SIGNATURES = {
     "br_plan_build_from_lengths": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "br_plan_build_packed": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "br_prefill_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
-    "br_prefill_workspace_bytes_fused": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "br_prefill_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "br_prefill_noalloc_max_workspace_bytes": (c_size_t, []),

@@ -337,7 +337,7 @@ def blockrank_attention(
     with torch.cuda.device(dev):
         plan = bm.plan(Nq, Nkv)
         out = torch.empty((Bt, S, Nq, D), dtype=query.dtype, device=dev)
-        ws_bytes = max(lib.br_prefill_workspace_bytes(B, Nq, Nkv, D), lib.br_prefill_workspace_bytes_fused(B, M, Nq, Nkv, D))
+        ws_bytes = lib.br_prefill_workspace_bytes(B, Nq, Nkv, D)
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         out_strides = _lib._I64x3(0 if packed else S * Nq * D, D, Nq * D)
         ev0, ev1 = kernel_events if kernel_events is not None else (None, None)

@@ -114,7 +114,7 @@ int check_strides(const char* name, const int64_t* s, int dtype) {
     return BR_OK;
 }
 
-size_t slots_total(int B, const BrGeom& g, int slots = BR_SLOTS_PER_SEQ) { return (size_t)B * slots * g.NHG; }
+size_t slots_total(int B, const BrGeom& g) { return (size_t)B * BR_SLOTS_PER_SEQ * g.NHG; }
 
 }  // namespace
 
@@ -179,14 +179,6 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     return rows * (size_t)(D + 2) * sizeof(float);
 }
 
-size_t br_prefill_workspace_bytes_fused(int B, int M, int Nq, int Nkv, int D) {
-    BrGeom g;
-    int nw;
-    if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || D <= 0 || M <= 0) return 0;
-    size_t rows = slots_total(B, g, br_slots_view1(M)) * (size_t)nw * BR_RB;
-    return rows * (size_t)(D + 2) * sizeof(float);
-}
-
 size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows) {
     if (B <= 0 || Nq <= 0 || M < 3 || H <= 0 || score_rows <= 0) return 0;
     return (size_t)B * Nq * score_rows * br_plan_tps(M, H) * 2 * sizeof(float);
@@ -236,16 +228,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
 
     BrPrefillParams p;
     p.q = q; p.k = k; p.v = v; p.out = out; p.plan = plan;
-    // The fused path (bf16: sequences of short blocks go to the resident kernel, the query block's rows are
-    // computed with each block) needs M-dependent room for partials.  It is opt-in for now - with
-    // BLOCKRANK_AMD_RESIDENT=1, and only when the caller's workspace has that room: on the measured
-    // workloads it does not beat the streaming kernel yet.
-    static const bool res_env = getenv("BLOCKRANK_AMD_RESIDENT") && atoi(getenv("BLOCKRANK_AMD_RESIDENT")) != 0;   // read once per process
-    const bool fused = dtype == BR_DTYPE_BF16 && fp8_tokens == 0 && !lse && (D == 64 || D == 128) && res_env &&
-                       workspace_bytes >= br_prefill_workspace_bytes_fused(B, M, Nq, Nkv, D);
-    p.queue_view = fused ? 1 : 0;
-    p.slots = fused ? br_slots_view1(M) : BR_SLOTS_PER_SEQ;
-    const size_t rows = slots_total(B, g, p.slots) * (size_t)nw * BR_RB;
+    const size_t rows = slots_total(B, g) * (size_t)nw * BR_RB;
     p.part_o = static_cast<float*>(workspace);
     p.part_ml = p.part_o + rows * D;
     p.sq_b = q_strides[0]; p.sq_h = q_strides[1]; p.sq_t = q_strides[2];
@@ -348,7 +331,6 @@ int br_prefill_fwd_noalloc(const void* q, const void* k, const void* v, void* ou
                                   "use br_prefill_fwd with a workspace, or a smaller batch", B, Nq, Nkv, D, need, (size_t)BR_NOALLOC_SCRATCH_BYTES);
     void* ws = nullptr;
     if ((rc = noalloc_scratch(&ws))) return rc;
-    // exactly `need` bytes are offered, so the call can never take the path that wants the larger (fused) workspace
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
                         ws, need, stream, nullptr, nullptr, 0, nullptr, 0);
 }
@@ -443,7 +425,7 @@ int br_prefill_bwd(const void* q, const void* k, const void* v, const void* out,
     p.geom = g;
     p.scale = scale;
     p.scale_log2 = scale * 1.4426950408889634f;
-    p.max_items = br_plan_max_items_view0(B, M, H, br_tokens_per_tile(g));
+    p.max_items = br_plan_max_items(B, M, H, br_tokens_per_tile(g));
     const int lrc = br_launch_bwd(p, D, nw, n_cu, static_cast<hipStream_t>(stream));
     if (lrc) return fail(BR_ERR_ARG, "no backward kernel for head dim %d with %d query heads per kv head (code %d)", D, g.G, lrc);
     return check_launch("backward launch");

@@ -8,7 +8,7 @@
 // over exactly the (query row, key) pairs the forward visits.  P is rebuilt from the log-sum-exp the forward
 // saved.  Two kernels, so that every sum that has one owner is kept in that owner's registers:
 //
-//   br_bwd_dq_kernel   query-major: walks the forward's own work items (view 0 of the request plan), one
+//   br_bwd_dq_kernel   query-major: walks the forward's own work items, one
 //                      workgroup per (item, head group), a wave per 32 rows of one query head.  Per 64-key tile
 //                      (K, V staged in LDS):  S^T = K Q^T, dP^T = V dO^T  (lane = query row, registers = keys)
 //                      -> dS^T in bf16 is directly the A operand of dQ += dS K (K through transposing LDS reads).
@@ -527,7 +527,7 @@ __global__ __launch_bounds__(MAXW * 64, MAXW <= 4 ? (D == 64 ? 3 : 2) : 1) void 
     const BrGeom& ge = p.geom;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
     const int item = blockIdx.x / ge.NHG, hg = blockIdx.x - item * ge.NHG;
-    if (item >= pv.hdr[BR_PH_QOFF2 + BR_GLOBAL_QUEUE]) return;      // view 0's items come first in the array; view 1 starts here
+    if (item >= pv.hdr[BR_PH_NITEMS]) return;
     const BrItem it = pv.items[item];
     Bwd<D>::dq_item(p, pv, it, hg, smem, blockDim.x >> 6);
 }

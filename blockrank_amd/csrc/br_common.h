@@ -17,10 +17,9 @@
 
 // Plan buffer (int32):
 //   [header BR_PLAN_HDR][start B*M][len B*M][tok B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
-//   [items 16*max_items][comb 4*2*max_comb][fused B]
-// The items array holds five groups: the query-block items (global queue) and the items of all other
-// blocks (XCD queues) of view 0, the same two of view 1 (without the fused sequences), and one
-// resident item per block of a fused sequence; the comb array holds view 0's entries, then view 1's.
+//   [items 16*max_items][comb 4*max_comb]
+// The items array holds the query-block items (global queue) followed by the items of all other blocks
+// (XCD queues).
 // Tile descriptors: for each sequence, the 64-key tiles of blocks 0..M-2 in order, as (token index of
 // the tile's first key, number of real keys); TPS = (M-1) * ceil(H/64) slots per sequence.
 // Work is handed out through 9 queues.  Queue 8 holds the query-block items (the long ones, with no
@@ -30,32 +29,21 @@
 // start at QOFF[g]); a ticket t of queue g is (item QOFF[g] + t / NHG, head group t % NHG):
 // consecutive tickets cover all kv heads, which keeps every L2 channel busy.
 #define BR_PLAN_HDR 96
-#define BR_RES_TILES 4          // the resident kernel keeps this many key/value tiles in LDS: a block's prefix tiles plus its own must fit
 #define BR_NQUEUES 9
 #define BR_GLOBAL_QUEUE 8
 enum BrPlanHeader {
     BR_PH_NITEMS = 0,     // number of work items (per head group)
     BR_PH_NCOMB = 1,      // number of combine entries (per head group)
     BR_PH_PACKED = 2,     // 1: tokens are packed (no padded slots between blocks), see tok[] below
-    BR_PH_NRES = 3,       // resident items: the blocks of the fused sequences
     BR_PH_NONCONTIG = 4,  // set to 1 if some block's real tokens are not one contiguous span
     BR_PH_MAX_ITEMS = 5,
     BR_PH_MAX_COMB = 6,
     BR_PH_T = 7,          // tokens per query tile the plan was built for
     BR_PH_QCOUNT = 8,     // [9] items in each queue
     BR_PH_QOFF = 17,      // [9] index of each queue's first item
-    BR_PH_RES_OFF = 26,   // index of the first resident item
-    BR_PH_NCOMB2 = 27,    // view 1: number of combine entries and index of the first one
-    BR_PH_COMB_OFF2 = 28,
-    BR_PH_SLOTS2 = 29,    // view 1: partial slots per sequence
     // second cache line: everything the running kernels update
     BR_PH_QTICKET = 32,   // [9] ticket counters (zero between launches)
-    BR_PH_RTICKET = 42,   // ticket counter of the resident kernel (zero between launches)
     BR_PH_DONE = 48,      // workgroups that have left the persistent loop (zero between launches)
-    BR_PH_RDONE = 49,     // the same for the resident kernel
-    // third cache line: the queues of view 1
-    BR_PH_QCOUNT2 = 64,   // [9]
-    BR_PH_QOFF2 = 73,     // [9]
 };
 
 // One unit of prefill work: query tile [t0, t0+T) of block m of sequence b, restricted to a range
@@ -97,17 +85,9 @@ __host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLA
 __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
     int qt = (H + T - 1) / T;
     int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
-    return B * (2 * ((M > 1 ? (M - 1) * qt : 0) + last) + M);
-}
-// Upper bound on the items of view 0 alone (they are the first items of the array).
-__host__ __device__ inline int br_plan_max_items_view0(int B, int M, int H, int T) {
-    int qt = (H + T - 1) / T;
-    int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
     return B * ((M > 1 ? (M - 1) * qt : 0) + last);
 }
-__host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }   // per view
-// Partial slots per sequence in view 1: a fused sequence uses (query tile, block) -> tile * M + block, two tiles at most.
-__host__ __device__ inline int br_slots_view1(int M) { return 2 * M > BR_SLOTS_PER_SEQ ? 2 * M : BR_SLOTS_PER_SEQ; }
+__host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }
 __host__ __device__ inline int br_plan_tps(int M, int H) { return (M > 1 ? M - 1 : 0) * ((H + BR_BN - 1) / BR_BN); }
 __host__ __device__ inline size_t br_plan_off_tbase(int B, int M) { return BR_PLAN_HDR + 3 * (size_t)B * M + (size_t)B; }
 __host__ __device__ inline size_t br_plan_off_tiles(int B, int M) { return (br_plan_off_tbase(B, M) + (size_t)B * M + 1) & ~(size_t)1; }
@@ -118,10 +98,9 @@ __host__ __device__ inline size_t br_plan_off_items(int B, int M, int H, int T) 
 __host__ __device__ inline size_t br_plan_off_comb(int B, int M, int H, int T) {
     return br_plan_off_items(B, M, H, T) + BR_ITEM_INTS * (size_t)br_plan_max_items(B, M, H, T);
 }
-__host__ __device__ inline size_t br_plan_off_fused(int B, int M, int H, int T) {
-    return br_plan_off_comb(B, M, H, T) + 4 * 2 * (size_t)br_plan_max_comb(B);
+__host__ __device__ inline size_t br_plan_total_ints(int B, int M, int H, int T) {
+    return br_plan_off_comb(B, M, H, T) + 4 * (size_t)br_plan_max_comb(B);
 }
-__host__ __device__ inline size_t br_plan_total_ints(int B, int M, int H, int T) { return br_plan_off_fused(B, M, H, T) + (size_t)B; }
 
 __device__ inline BrPlanView br_plan_view(const int* plan, int B, int M, int H, int T) {
     BrPlanView v;
@@ -175,15 +154,6 @@ __device__ inline void br_leave(int* hdr) {
     if (d == (int)gridDim.x - 1) {
         for (int i = 0; i < BR_NQUEUES; ++i) atomicExch(&hdr[BR_PH_QTICKET + i], 0);
         atomicExch(&hdr[BR_PH_DONE], 0);
-    }
-}
-
-// The same for the resident kernel.
-__device__ inline void br_leave_resident(int* hdr) {
-    int d = atomicAdd(&hdr[BR_PH_RDONE], 1);
-    if (d == (int)gridDim.x - 1) {
-        atomicExch(&hdr[BR_PH_RTICKET], 0);
-        atomicExch(&hdr[BR_PH_RDONE], 0);
     }
 }
 
@@ -286,10 +256,6 @@ struct BrPrefillParams {
     const float* qk_scales;
     const void* k8;
     unsigned k8_b, k8_h;
-    // 0: every sequence goes through the streaming kernel; 1: the plan's second view, in which the
-    // fused sequences are left to the resident kernel
-    int queue_view;
-    int slots;         // partial slots per sequence (BR_SLOTS_PER_SEQ in view 0, br_slots_view1(M) in view 1)
     // Optional: the log-sum-exp of every real query row, in base-2 units (log2 of the sum over the visible keys
     // of 2^(scale * log2(e) * q.k)), at lse[b * lse_b + head * lse_h + token]; the backward pass starts from it.
     // Null: not wanted.  Written by the streaming bf16 kernel and the finish kernel only.

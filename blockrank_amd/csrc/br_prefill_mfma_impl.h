@@ -72,6 +72,18 @@ __device__ inline bf16x8 as_bf16x8(uint4 u) {
     return c.v;
 }
 __device__ inline int uni(int x) { return __builtin_amdgcn_readfirstlane(x); }
+// The value of lane ^ 32 combined with the lane's own: one v_permlane32_swap (which exchanges the upper half of its
+// first operand with the lower half of its second) instead of a trip through the LDS crossbar.
+__device__ inline float max_xor32(float x) {
+    const unsigned u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+// Scheduling directives for the compiler's instruction scheduler: a group of `n` instructions of one kind, placed in
+// the order the directives are written; unmatched instructions go where their dependencies allow.
+#define BR_SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
+#define BR_SCHED_DSREAD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
+#define BR_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 // 64 lanes x 16 bytes from global memory (uniform base + per-lane byte offset) into LDS at
 // lds_addr + lane * 16.  Issued through asm so that the compiler does not make later LDS reads of
@@ -150,11 +162,10 @@ struct BrPrefetch {
     // the queue blockIdx & 7 (workgroups are dealt round robin to the XCDs, so this is normally the
     // queue of the XCD they run on; if it is not, only locality is lost).  The counters therefore
     // count the tickets drawn after the static ones.
-    __device__ void init(int* hdr_, const BrPlanView* pv_, int NHG_, int lane_, int view) {
+    __device__ void init(int* hdr_, const BrPlanView* pv_, int NHG_, int lane_) {
         hdr = hdr_; pv = pv_; NHG = NHG_; lane = lane_;
-        const bool v1 = view == 1;
-        counts = lane < BR_NQUEUES ? hdr[(v1 ? BR_PH_QCOUNT2 : BR_PH_QCOUNT) + lane] * NHG : 0;
-        qoffs = lane < BR_NQUEUES ? hdr[(v1 ? BR_PH_QOFF2 : BR_PH_QOFF) + lane] : 0;
+        counts = lane < BR_NQUEUES ? hdr[BR_PH_QCOUNT + lane] * NHG : 0;
+        qoffs = lane < BR_NQUEUES ? hdr[BR_PH_QOFF + lane] : 0;
         const int grid = gridDim.x, me = blockIdx.x;
         // Queue ownership goes by workgroup index, not by the XCD id the hardware reports: every queue
         // then has its workgroups whatever the placement is, so all work is done in any case.
@@ -437,6 +448,16 @@ struct Prefill {
                 if (i + 4 < NR) ka[i & 3] = read_k(stage, L, (i + 4) % NKB, (i + 4) / NKB);
                 s[i % NKB] = mma_qk(a, qf[i / NKB], s[i % NKB]);
             }
+            // keep that order: four operand reads in flight ahead of every product (left alone, the scheduler
+            // shortens the live ranges until every product waits for its own read)
+            BR_SCHED_DSREAD(4);
+#pragma unroll
+            for (int i = 0; i + 4 < NR; ++i) {
+                BR_SCHED_MFMA(1);
+                BR_SCHED_DSREAD(1);
+            }
+            BR_SCHED_MFMA(4);
+            BR_SCHED_FENCE();
         }
         // first V^T operands: their LDS latency passes under the softmax arithmetic
         bf16x8 va[ND];
@@ -456,7 +477,7 @@ struct Prefill {
         for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = max_xor32(mx);
         // Lazy rescale: the running max is only raised (and O, l rescaled) when some row's max grew by
         // more than 2^8; otherwise exponentials are taken against the older max, which changes nothing
         // in the final quotient and keeps them below 2^8.
@@ -718,7 +739,7 @@ struct Prefill {
         const float lt_tot = lt_run + __shfl_xor(lt_run, 32);    // sum of the rounded probabilities: normalises the output
         if (it.slot >= 0) {
             if (row0 + ln < len_m) {
-                const long long slot = ((long long)b * p.slots + it.slot) * ge.NHG + hg;
+                const long long slot = ((long long)b * BR_SLOTS_PER_SEQ + it.slot) * ge.NHG + hg;
                 const long long prow = slot * (NW * BR_RB) + wave * BR_RB + ln;
                 float* po = p.part_o + prow * D;
 #pragma unroll
@@ -796,13 +817,6 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
     const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    {   // nothing queued at all (every sequence went to the resident kernel): leave at once
-        const int c = lane < BR_NQUEUES ? hdr[(p.queue_view == 1 ? BR_PH_QCOUNT2 : BR_PH_QCOUNT) + lane] : 0;
-        if (__builtin_amdgcn_ballot_w64(c > 0) == 0) {
-            if (threadIdx.x == 0) br_leave(hdr);
-            return;
-        }
-    }
     const typename PF::Lane L = PF::make_lane(p, wave, lane);
     // fp8 kernel: the query block's items (the rows the document scores are read from, and the single block of a
     // sequence without documents) run on the bf16 Q and K, every other item on the e4m3 copies
@@ -822,7 +836,7 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     for (int i = threadIdx.x * 16; i < Smem<D, F8>::total(NW); i += NW * 64 * 16) *reinterpret_cast<uint4*>(smem + i) = uint4{0u, 0u, 0u, 0u};
     const bool padded_layout = uni(hdr[BR_PH_PACKED]) == 0;
     BrPrefetch pf;
-    pf.init(hdr, &pv, NHG, lane, p.queue_view);
+    pf.init(hdr, &pv, NHG, lane);
     if (wave == 0) pf.publish(&mail[0]);
     __syncthreads();
     for (int cur = 0;; cur ^= 1) {
@@ -850,284 +864,6 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
     if (threadIdx.x == 0) br_leave(hdr);
 }
 
-// Resident variant for the fused sequences (short blocks): one workgroup of eight waves takes
-// (block, head group), loads every key/value tile the block's rows can see - the prefix's tiles and
-// the block's own, at most BR_RES_TILES - into LDS once, and then its waves work through row blocks
-// (32 rows of one head each, handed out through an LDS counter, the block's own rows with the longest
-// walk first) independently of each other: no barrier, no load and no bookkeeping per tile, and the
-// set-up of one wave's row block (its Q rows, its output stores) runs under the arithmetic of the
-// other waves.  The query block's rows are row blocks of every item too: against the keys of this
-// block they give an unnormalised partial (slot: query tile * M + block), merged by the finish
-// kernel, and - for a document - the score partials of the block's tiles.  K/V are thus read once.
-template <int D>
-struct Resident {
-    static constexpr int NW = 8;
-    using PF = Prefill<D, NW, false>;
-    using SM = Smem<D, false>;
-    using Lane = typename PF::Lane;
-    static constexpr int kStageBytes = BR_RES_TILES * SM::stageBytes;
-    static constexpr int kCtlInts = 32;
-    static constexpr int kLdsBytes = kStageBytes + kCtlInts * 4;
-
-    // One row block: rows [row0, row0+32) of `head`, taken from the block of q_len tokens that starts at
-    // token q_tok, against the tiles (LDS stages) [f_lo, f_hi).  Stages below n0 hold the prefix (len0
-    // keys), the others the item's own block (len_m keys); with `causal` the own keys obey the causal
-    // rule.  slot < 0: normalised output rows; else: partial into that slot (row block `wave4` of it).
-    // qf: the row block's Q^T fragments, in registers; qn: those of the wave's next row block, in flight.
-    //
-    // (load_q) Requests the Q^T fragments of a row block: lane (ln, lh) holds row row0+ln, dims 16c + 8lh .. +7 of chunk c.
-    static __device__ __forceinline__ void load_q(const BrPrefillParams& p, int b, int head, int q_tok, int q_len, int row0, int lane,
-                                                  typename PF::Frag (&qf)[D / 16]) {
-        const int ln = lane & 31, lh = lane >> 5;
-        const char* qrow = reinterpret_cast<const char*>(p.q) +
-                           ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)head +
-                            (unsigned long long)p.q32_t * (unsigned)(q_tok + row0)) * 2;
-        const int last = q_len - 1 - row0;       // rows past the block's end load its last row; they are never stored
-        const int qoff = ((ln < last ? ln : last) * (int)p.q32_t + lh * 8) * 2;
-#pragma unroll
-        for (int c = 0; c < D / 16; ++c) qf[c] = as_bf16x8(ld16(qrow + qoff + c * 32));
-    }
-
-    static __device__ __forceinline__ void row_block(const BrPrefillParams& p, const BrPlanView& pv, const BrItem& it, int b, int hg, int head, int q_tok,
-                                     int q_len, int row0, int n0, int f_lo, int f_hi, bool causal, int slot, int wave4, bool scores,
-                                     const char* smem, const Lane& L, int lane, const typename PF::Frag (&qf)[D / 16],
-                                     typename PF::Frag (&qn)[D / 16]) {
-        const int ln = lane & 31, lh = lane >> 5;
-        f32x16 o[D / 32];
-#pragma unroll
-        for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o[d][v] = 0.f;
-        float m_run = -INFINITY, l_run = 0.f, lt_run = 0.f;
-
-        for (int f = f_lo; f < f_hi; ++f) {
-            const char* stage = smem + f * SM::stageBytes;
-            const bool prev = f < n0;
-            const int key0 = (f - n0) * BR_BN;
-            int nv = prev ? it.len0 - f * BR_BN : it.len_m - key0;
-            nv = nv < BR_BN ? nv : BR_BN;
-            // (per-lane copies of the tile quantities: see run_item)
-            int v_nvalid = nv, v_self = (!prev && causal) ? 1 : 0, v_key0 = key0;
-            asm volatile("" : "+v"(v_nvalid), "+v"(v_self), "+v"(v_key0));
-            int nkb = (v_nvalid + 31) >> 5;
-            const bool c_self = v_self != 0;
-            if (c_self) {
-                int vis = row0 + BR_RB - v_key0;
-                int c = vis <= 0 ? 0 : (vis + 31) >> 5;
-                nkb = c < nkb ? c : nkb;
-            }
-            const bool need_mask = (v_nvalid < nkb * 32) || (c_self && v_key0 + nkb * 32 - 1 > row0);
-            float psum = 0.f;
-            if (nkb == 2 && !need_mask) {
-                PF::template compute_tile<2, false>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, 0, lh, psum);
-            } else if (nkb > 0) {
-                const int lim_causal = c_self ? row0 + ln - v_key0 + 1 : BR_BN;
-                const int lim = v_nvalid < lim_causal ? v_nvalid : lim_causal;
-                if (nkb == 2) PF::template compute_tile<2, true>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, lim, lh, psum);
-                else if (need_mask) PF::template compute_tile<1, true>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, lim, lh, psum);
-                else PF::template compute_tile<1, false>(stage, L, qf, o, m_run, l_run, lt_run, p.scale_log2, lim, lh, psum);
-            }
-            if (scores) {
-                // this tile's probability mass (against the running max) for the query block's last rows
-                int lane_s = lane;
-                asm volatile("" : "+v"(lane_s));
-                const float tot = psum + __shfl_xor(psum, 32);
-                const int ln_s = lane_s & 31;
-                const int r16 = it.slot + row0 + ln_s - (p.H - p.score_R);
-                if (lane_s < 32 && r16 >= 0 && row0 + ln_s < q_len) {
-                    float2 ms = make_float2(m_run == -INFINITY ? 0.f : m_run, tot);
-                    *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + it.ntiles + (f - n0)) * 2) = ms;
-                }
-            }
-        }
-
-        // the next row block's Q rows were requested before this one's arithmetic: they are here by now, and
-        // nothing else is in flight but older stores, so this wait costs nothing (taken before this row
-        // block's stores are issued, it does not wait for them either)
-        vm_wait_all();
-#pragma unroll
-        for (int c = 0; c < D / 16; ++c) asm volatile("" : "+v"(qn[c]));
-
-        int lane_e = lane;
-        asm volatile("" : "+v"(lane_e));
-        const int ln_e = lane_e & 31, lh_e = lane_e >> 5;
-        const float l_tot = lt_run + __shfl_xor(lt_run, 32);     // sum of the rounded probabilities (see compute_tile)
-        (void)l_run;
-        const bool ok = row0 + ln_e < q_len;
-        if (slot >= 0) {
-            if (ok) {
-                const long long sidx = ((long long)b * p.slots + slot) * p.geom.NHG + hg;
-                const long long prow = sidx * (p.geom.Gw * p.geom.tpb * BR_RB) + wave4 * BR_RB + ln_e;
-                float* po = p.part_o + prow * D;
-#pragma unroll
-                for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        f32x4 t = {o[d][4 * q4], o[d][4 * q4 + 1], o[d][4 * q4 + 2], o[d][4 * q4 + 3]};
-                        *reinterpret_cast<f32x4*>(po + d * 32 + 8 * q4 + 4 * lh_e) = t;
-                    }
-                if (lh_e == 0) {
-                    p.part_ml[prow * 2] = m_run;
-                    p.part_ml[prow * 2 + 1] = l_tot;
-                }
-            }
-            return;
-        }
-        // Epilogue without LDS: lane (ln, lh) holds, of row row0+ln, dims 32d + 8j + 4lh + 0..3 (j = 0..3).
-        // Exchanging the odd-j pieces of the lower lane half with the even-j pieces of the upper half
-        // gives every lane whole 16-byte pieces: dims 32d + 16e + 8lh + 0..7 (e = 0, 1).
-        const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;
-        char* orow = reinterpret_cast<char*>(p.out) +
-                     2 * ((unsigned long long)p.o32_b * (unsigned)b + (unsigned long long)p.o32_h * (unsigned)head +
-                          (unsigned long long)p.o32_t * (unsigned)(q_tok + row0 + ln_e) + lh_e * 8);
-#pragma unroll
-        for (int d = 0; d < D / 32; ++d)
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                union { bf16x4 h; unsigned u[2]; } ev, od;
-                f32x4 te = {o[d][8 * e] * inv, o[d][8 * e + 1] * inv, o[d][8 * e + 2] * inv, o[d][8 * e + 3] * inv};
-                f32x4 to = {o[d][8 * e + 4] * inv, o[d][8 * e + 5] * inv, o[d][8 * e + 6] * inv, o[d][8 * e + 7] * inv};
-                ev.h = __builtin_convertvector(te, bf16x4);
-                od.h = __builtin_convertvector(to, bf16x4);
-                auto s0 = __builtin_amdgcn_permlane32_swap(ev.u[0], od.u[0], false, false);
-                auto s1 = __builtin_amdgcn_permlane32_swap(ev.u[1], od.u[1], false, false);
-                uint4 val = {s0[0], s1[0], s0[1], s1[1]};
-                if (ok) *reinterpret_cast<uint4*>(orow + (d * 32 + e * 16) * 2) = val;
-            }
-    }
-};
-
-template <int D>
-__global__ __launch_bounds__(512, 1) void br_prefill_resident_kernel(BrPrefillParams p) {
-    extern __shared__ __attribute__((aligned(1024))) char rsmem[];
-    using R = Resident<D>;
-    using PF = typename R::PF;
-    using SM = typename R::SM;
-    int* ctl = reinterpret_cast<int*>(rsmem + R::kStageBytes);     // [0] row-block counter, [1] next ticket
-    const BrGeom& ge = p.geom;
-    const int NHG = ge.NHG;
-    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
-    int* hdr = const_cast<int*>(p.plan);
-    const int wave = uni(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int n_tickets = hdr[BR_PH_NRES] * NHG;
-    if ((int)blockIdx.x >= n_tickets) {       // no item for this workgroup (none at all when no sequence is fused)
-        if (threadIdx.x == 0) br_leave_resident(hdr);
-        return;
-    }
-    const typename PF::Lane L = PF::make_lane(p, wave, lane);
-    // DMA pieces of partial tiles are skipped, so whatever sits in LDS must be finite: start from zero
-    for (int i = threadIdx.x * 16; i < R::kStageBytes; i += 512 * 16) *reinterpret_cast<uint4*>(rsmem + i) = uint4{0u, 0u, 0u, 0u};
-    const int res_off = hdr[BR_PH_RES_OFF];
-    const unsigned smem_lds = lds_addr_of(rsmem);
-    const int sk_bytes = (int)p.k32_t * 2, sv_bytes = (int)p.v32_t * 2;
-    const int T = ge.tpb * BR_RB;
-    const float inv_gw = 1.0f / (float)ge.Gw;
-    // the first ticket of a workgroup is its index; later ones come from the counter
-    int ticket = blockIdx.x;
-    __syncthreads();
-    while (ticket < n_tickets) {
-        const int li = ticket / NHG, hg = ticket - li * NHG;
-        int w = 0;
-        if (lane < BR_ITEM_INTS) w = reinterpret_cast<const int*>(pv.items + res_off + li)[lane];
-        int t_next = 0;
-        if (threadIdx.x == 0) {
-            t_next = atomicAdd(&hdr[BR_PH_RTICKET], 1);
-            ctl[0] = 0;
-        }
-        BrItem it;
-#define BR_W(i) __builtin_amdgcn_readlane(w, i)
-        it.b = BR_W(0); it.m = BR_W(1); it.t0 = BR_W(2); it.f_lo = BR_W(3); it.nprev = BR_W(4); it.ntiles = BR_W(5); it.slot = BR_W(6);
-        it.pe = BR_W(7); it.len_m = BR_W(8); it.start_m = BR_W(9); it.len0 = BR_W(10); it.start0 = BR_W(11); it.tok_m = BR_W(12);
-        it.tok0 = BR_W(13);
-        it.pad[0] = it.pad[1] = 0;
-#undef BR_W
-        const int b = it.b, m = it.m;
-        const bool is_q = m == p.M - 1;
-        const int q_len = it.t0, q_tok = it.f_lo;               // the query block's span (see the plan)
-        const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
-        const int n0 = it.nprev, n1 = (it.len_m + BR_BN - 1) / BR_BN;
-        const char* kbase = reinterpret_cast<const char*>(p.k) + ((unsigned long long)p.k32_b * (unsigned)b + (unsigned long long)p.k32_h * (unsigned)kvh) * 2;
-        const char* vbase = reinterpret_cast<const char*>(p.v) + ((unsigned long long)p.v32_b * (unsigned)b + (unsigned long long)p.v32_h * (unsigned)kvh) * 2;
-        {
-            int lane_l = lane;
-            asm volatile("" : "+v"(lane_l));
-            for (int f = 0; f < n0 + n1; ++f) {
-                const bool prev = f < n0;
-                const int k0 = (f - n0) * BR_BN;
-                const int tok = prev ? it.tok0 + f * BR_BN : it.tok_m + k0;
-                int nv = prev ? it.len0 - f * BR_BN : it.len_m - k0;
-                nv = nv < BR_BN ? nv : BR_BN;
-                PF::issue_tile(L, wave, lane_l, kbase + (long long)tok * sk_bytes, vbase + (long long)tok * sv_bytes, sk_bytes, sv_bytes, nv,
-                               smem_lds + f * SM::stageBytes);
-            }
-        }
-        vm_wait_all();
-        __syncthreads();
-        const int nT = (it.len_m + BR_RB - 1) / BR_RB;
-        const int n_own = is_q ? 0 : nT * ge.Gw;
-        const int nrb = n_own + ((q_len + BR_RB - 1) / BR_RB) * ge.Gw;
-        const int head0 = kvh * ge.G + hsub * ge.Gw;
-        // a row block as scalars: head, the block its rows come from, the tiles it walks, where its result goes
-        int c_head = 0, c_tok = 0, c_len = 0, c_row0 = 0, c_flo = 0, c_fhi = 0, c_causal = 0, c_slot = -1, c_w4 = 0, c_sc = 0;
-        int n_head = 0, n_tok = 0, n_len = 0, n_row0 = 0, n_flo = 0, n_fhi = 0, n_causal = 0, n_slot = -1, n_w4 = 0, n_sc = 0;
-        // Order: the query block's row blocks first (as long a walk as any, and the biggest epilogue), then the
-        // block's own from the last (longest walk) to the first.  Index -> (32-row block, head) without
-        // integer division: the quotients are tiny, a float multiply is exact for them.
-        const int n_qrb = ((q_len + BR_RB - 1) / BR_RB) * ge.Gw;
-        auto draw = [&]() -> bool {
-            int r = 0;
-            if (lane == 0) r = atomicAdd(&ctl[0], 1);
-            r = uni(r);
-            if (r >= nrb) return false;
-            const bool own = r >= n_qrb;
-            const int rr = own ? r - n_qrb : r;
-            const int blk = uni((int)(((float)rr + 0.5f) * inv_gw));
-            const int g = rr - blk * ge.Gw;
-            n_head = head0 + g;
-            if (own) {
-                n_row0 = (nT - 1 - blk) * BR_RB;
-                const int row_end = n_row0 + BR_RB < it.len_m ? n_row0 + BR_RB : it.len_m;
-                n_tok = it.tok_m; n_len = it.len_m;
-                n_flo = 0; n_fhi = n0 + ((row_end + BR_BN - 1) >> 6);
-                n_causal = 1; n_slot = -1; n_w4 = 0; n_sc = 0;
-            } else {
-                n_row0 = blk * BR_RB;
-                const int tq = n_row0 >= T ? 1 : 0;            // a fused sequence's query block has at most two query tiles
-                const int sub = (n_row0 - tq * T) >> 5;
-                const int row_end = n_row0 + BR_RB < q_len ? n_row0 + BR_RB : q_len;
-                n_tok = q_tok; n_len = q_len;
-                n_flo = n0; n_fhi = is_q ? ((row_end + BR_BN - 1) >> 6) : n0 + n1;
-                n_causal = is_q ? 1 : 0; n_slot = tq * p.M + m; n_w4 = g * ge.tpb + sub;
-                n_sc = (p.score_part != nullptr && !is_q && m >= 1) ? 1 : 0;
-            }
-            return true;
-        };
-        typename PF::Frag qf[D / 16], qn[D / 16];
-        bool have = draw();
-        if (have) {
-            R::load_q(p, b, n_head, n_tok, n_len, n_row0, lane, qn);
-            vm_wait_all();
-#pragma unroll
-            for (int c = 0; c < D / 16; ++c) asm volatile("" : "+v"(qn[c]));
-        }
-        while (have) {
-#pragma unroll
-            for (int c = 0; c < D / 16; ++c) qf[c] = qn[c];
-            c_head = n_head; c_tok = n_tok; c_len = n_len; c_row0 = n_row0; c_flo = n_flo; c_fhi = n_fhi;
-            c_causal = n_causal; c_slot = n_slot; c_w4 = n_w4; c_sc = n_sc;
-            // the next row block's Q rows travel while this one is computed
-            have = draw();
-            if (have) R::load_q(p, b, n_head, n_tok, n_len, n_row0, lane, qn);
-            R::row_block(p, pv, it, b, hg, c_head, c_tok, c_len, c_row0, n0, c_flo, c_fhi, c_causal != 0, c_slot, c_w4, c_sc != 0, rsmem, L, lane,
-                         qf, qn);
-        }
-        if (threadIdx.x == 0) ctl[1] = (int)gridDim.x + t_next;
-        __syncthreads();
-        ticket = uni(ctl[1]);
-    }
-    if (threadIdx.x == 0) br_leave_resident(hdr);
-}
-
 // Finish: (1) merge the split-KV partials of the query block,
 // out = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m); one workgroup per (query tile, head group, row
 // block); (2) set the rows of padded token slots to zero.
@@ -1138,8 +874,8 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
     constexpr int CPR = D / 4;                    // float4 chunks per row = threads per row
     constexpr int RPW = 256 / CPR;                // rows one workgroup merges at a time
     constexpr int SUBS = BR_RB / RPW;             // such row groups per 32-row block
-    const int n_units = pv.hdr[p.queue_view == 1 ? BR_PH_NCOMB2 : BR_PH_NCOMB] * ge.NHG * NW * SUBS;
-    const BrComb* combs = pv.comb + (p.queue_view == 1 ? pv.hdr[BR_PH_COMB_OFF2] : 0);
+    const int n_units = pv.hdr[BR_PH_NCOMB] * ge.NHG * NW * SUBS;
+    const BrComb* combs = pv.comb;
     const int m = p.M - 1;
     const int rows = NW * BR_RB;
     const int rr = threadIdx.x / CPR, cc = threadIdx.x % CPR;
@@ -1158,7 +894,7 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
         if (row >= len_m) continue;
         const int head = kvh * ge.G + hsub * ge.Gw + g;
         const int r = wave * BR_RB + rloc;
-        const long long slot0 = ((long long)c.b * p.slots + c.slot0) * ge.NHG + hg;
+        const long long slot0 = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0) * ge.NHG + hg;
         const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
         const float2* ml = reinterpret_cast<const float2*>(p.part_ml) + slot0 * rows + r;
         const float* po = p.part_o + (slot0 * rows + r) * D + cc * 4;
@@ -1196,17 +932,15 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
         bf16x4 h4 = __builtin_convertvector(acc * inv, bf16x4);
         *reinterpret_cast<bf16x4*>(dst + cc * 4) = h4;
     }
-    // Padded token slots: no kernel computes them, so give them a defined value (zero).  The prefill kernels
-    // streaming kernel does that for the documents it has items for; what is left here are the prefix and
-    // the query block, documents with no real token at all, and the blocks of the fused sequences, which the
-    // resident kernel computes (a packed layout has no padded slots).
-    const int* fused = p.plan + br_plan_off_fused(p.B, p.M, p.H, ge.tpb * BR_RB);
+    // Padded token slots: no kernel computes them, so give them a defined value (zero).  The prefill kernel
+    // does that for the documents it has items for; what is left here are the prefix, the query block and
+    // documents with no real token at all (a packed layout has no padded slots).
     const int n_pad_work = pv.hdr[BR_PH_PACKED] ? 0 : p.B * p.M * p.Nq;
     for (int w = blockIdx.x; w < n_pad_work; w += gridDim.x) {
         const int bm = w / p.Nq, head = w - bm * p.Nq;
         const int b = bm / p.M, mm = bm - b * p.M;
         const int st = pv.start[bm], ln = pv.len[bm];
-        if (ln != 0 && mm > 0 && mm < p.M - 1 && !(p.queue_view == 1 && fused[b] != 0)) continue;
+        if (ln != 0 && mm > 0 && mm < p.M - 1) continue;
         const int npad = p.H - ln;
         constexpr int CP8 = D / 8;
         __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;

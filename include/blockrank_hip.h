@@ -74,14 +74,6 @@ int br_plan_build_packed(const int32_t* lens, int B, int M, int H, int Nq, int N
 /* Bytes of scratch br_prefill_fwd needs (split-KV partials of the query block). */
 size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D);
 
-/* Bytes of scratch that let the bf16 entry points take the fused path for sequences of short blocks
- * (every block's keys, with the prefix's, fit in LDS: one workgroup then computes the block's rows
- * and the query block's rows against it, and K/V are read once).  Never less than
- * br_prefill_workspace_bytes; with a smaller workspace the entry points use the streaming kernel for
- * everything.  No reference counterpart (the reference computes the three groups of rows with three
- * SDPA calls, blockrank_std_attention.py:556-629). */
-size_t br_prefill_workspace_bytes_fused(int B, int M, int Nq, int Nkv, int D);
-
 /* Block-sparse prefill attention.  Replaces sdpa_blockrank_attention_forward /
  * eager_blockrank_attention_forward (blockrank_std_attention.py:472-650, :96-262) and
  * triton_blockrank_attention_forward (blockrank_triton_kernel_attention.py:798-884) including their

@@ -43,9 +43,6 @@ def test_pure_host_entry_points():
     assert lib.br_plan_ints(0, 22, 160, 32, 8) == 0
     assert lib.br_prefill_workspace_bytes(4, 32, 8, 128) == 4 * 32 * 8 * 128 * 130 * 4
     assert lib.br_doc_scores_workspace_bytes(4, 32, 22, 2) == 4 * 32 * 2 * 20 * 2 * 4
-    # the fused path keeps one partial slot per (query tile, block): 2 * M slots, never fewer than the 32 of the split path
-    assert lib.br_prefill_workspace_bytes_fused(4, 22, 32, 8, 128) == 4 * 44 * 8 * 128 * 130 * 4
-    assert lib.br_prefill_workspace_bytes_fused(4, 5, 32, 8, 128) == lib.br_prefill_workspace_bytes(4, 32, 8, 128)
     assert lib.br_prefill_fp8qk_workspace_bytes(4, 32, 8, 128, 4 * 3520) > lib.br_prefill_workspace_bytes(4, 32, 8, 128)
     # backward: fp32 sums of the query block's dQ rows and of the prefix keys' dK / dV, rounded up to 256 bytes, then one
     # float per token slot and query head (delta)

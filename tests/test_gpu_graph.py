@@ -12,9 +12,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("resident", ["0", "1"])
-def test_graph_replays_equal_eager(resident, monkeypatch):
-    monkeypatch.setenv("BLOCKRANK_AMD_RESIDENT", resident)
+def test_graph_replays_equal_eager():
     lay = synthetic.make_layout([[40, 100, 160, 33, 192, 20], [64, 7, 150, 90, 0, 31]])
     Nq, Nkv, D = 8, 2, 128
     scale = D ** -0.5
