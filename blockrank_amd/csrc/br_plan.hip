@@ -10,6 +10,9 @@
 namespace {
 
 constexpr int kPlanThreads = 1024;
+#ifndef BR_TILE_ORDER_DESC
+#define BR_TILE_ORDER_DESC 1
+#endif
 
 // One wave per block: count real tokens, find the first and the last.  len is written negated
 // (-1 - count) when the real tokens are not one contiguous span; the plan kernel repairs the sign
@@ -231,13 +234,16 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             it.pad[0] = it.pad[1] = 0;
             if (!is_last) {
                 it.nprev = npt;
-                for (int tt = 0; tt < nq; ++tt) {
+                // a block's query tiles are handed out from the last (the longest walk) to the first: what a queue
+                // ends on are short items
+                for (int k = 0; k < nq; ++k) {
+                    const int tt = BR_TILE_ORDER_DESC ? nq - 1 - k : k;
                     it.t0 = tt * T; it.f_lo = 0;
                     it.ntiles = 0x7fffffff; it.slot = -1;
-                    items[off_x + tt] = it;
+                    items[off_x + k] = it;
                     int q = w_total > 0 ? (int)(off_w * 8 / w_total) : 0;
                     q = q > 7 ? 7 : q;
-                    atomicMin(&s_qfirst[q], off_x + tt);
+                    atomicMin(&s_qfirst[q], off_x + k);
                     off_w += item_weight(npt, tt, L);
                 }
             } else {

@@ -428,7 +428,7 @@ struct Prefill {
     // NKB 32-key halves are computed (the second half is skipped when no row of the wave can see it);
     // with MASK, keys >= lim (per row: the tile's real keys and the diagonal) are excluded.  Every
     // variant is one straight-line block with the LDS operand reads issued ahead of their use.
-    template <int NKB, bool MASK>
+    template <int NKB, bool MASK, bool EXACT>
     static __device__ inline void compute_tile(const char* stage, const Lane& L, const Frag (&qf)[D / 16], f32x16 (&o)[D / 32],
                                                float& m_run, float& l_run, float& lt_run, float scale_log2, int lim, int lh, float& psum_out) {
         constexpr int NC = D / 16, ND = D / 32, NR = NKB * NC;
@@ -507,7 +507,7 @@ struct Prefill {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 t[e] = __builtin_amdgcn_exp2f(s[c2 >> 1][8 * (c2 & 1) + e] * scale_log2 - m_sub);
-                psum += t[e];
+                if (EXACT) psum += t[e];
             }
             pf[c2] = __builtin_convertvector(t, bf16x8);
             psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 0, 1), ones2, psum_t, false);
@@ -568,6 +568,7 @@ struct Prefill {
         const bool table = it.pe > 1;
         // only query-block items of a sequence with documents emit score partials, for document tiles
         const bool emit_scores = p.score_part != nullptr && table && m == p.M - 1;
+        const bool exact = emit_scores || p.lse != nullptr;
         const int first_doc_tile = (it.len0 + BR_BN - 1) / BR_BN;
         const int nprev = it.nprev;
         const int f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
@@ -701,14 +702,24 @@ struct Prefill {
             if (!rb_active) nkb = 0;
             const bool need_mask = (v_nvalid < nkb * 32) || (c_self && key0 + nkb * 32 - 1 > row0);
             float psum = 0.f;
-            if (nkb == 2 && !need_mask) {
-                compute_tile<2, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, 0, lh, psum);
-            } else if (nkb > 0) {
+            // (the exact sum of the probabilities is only kept where something reads it: the log-sum-exp output and
+            // the score partials; everything else normalises by the sum of the rounded values alone)
+            if (nkb > 0) {
                 const int lim_causal = c_self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
                 const int lim = v_nvalid < lim_causal ? v_nvalid : lim_causal;
-                if (nkb == 2) compute_tile<2, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
-                else if (need_mask) compute_tile<1, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
-                else compute_tile<1, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                int v_exact = exact ? 1 : 0;                 // (a per-lane value, like the tile quantities above)
+                asm volatile("" : "+v"(v_exact));
+                if (v_exact != 0) {
+                    if (nkb == 2 && !need_mask) compute_tile<2, false, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, 0, lh, psum);
+                    else if (nkb == 2) compute_tile<2, true, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                    else if (need_mask) compute_tile<1, true, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                    else compute_tile<1, false, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                } else {
+                    if (nkb == 2 && !need_mask) compute_tile<2, false, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, 0, lh, psum);
+                    else if (nkb == 2) compute_tile<2, true, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                    else if (need_mask) compute_tile<1, true, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                    else compute_tile<1, false, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                }
             }
             // Score partials: this tile's probability mass (against the running max) for the query block's
             // last rows, per head - everything the per-document scores need, with no second pass over K.
