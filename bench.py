@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BlockRank attention + per-document score path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5shape|cfg1] [--qk-fp8] [--backward] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5shape|cfg1] [--qk-fp8] [--backward] [--no-cpu-baseline] [--no-e2e]
 
 A step is one pass of the hot path over one batch already resident in HBM: the attention hook
 (block-sparse prefill attention of one layer, query/key/value as a Mistral layer hands them over)
@@ -21,7 +21,10 @@ Prints ONE JSON line: requests/s for the batch, plus
   roofline_hbm  the same kernel against the HBM peak (algorithmic bytes: Q, K, V read once, O
                 written once) - the op sits below the machine ridge, so this roof co-binds;
   cpu_baseline  the CPU restatement of the reference's three-call SDPA algorithm + score formula,
-                timed on this machine's host cores on a bounded sample (one sequence of the batch).
+                timed on this machine's host cores on a bounded sample (one sequence of the batch);
+  e2e           (default workload) the whole ranking request measured in the same run: the --workload cfg3 forward,
+                five batches - requests/s, ms per batch, the attention launches' share and roofline fraction, the
+                plan's cost.
 """
 from __future__ import annotations
 
@@ -136,8 +139,9 @@ def cpu_baseline_backward(layout, q, k, v, dout, scale, dtype, budget_s=12.0):
                 ms_per_sequence=med * 1e3)
 
 
-def bench_model(args):
-    """cfg3: the truncated ranking forward of a Mistral-7B-shaped model with random weights."""
+def run_model(args, steps, warmup):
+    """cfg3: the truncated ranking forward of a Mistral-7B-shaped model with random weights.  Returns the result
+    line as a dict."""
     import blockrank_amd as br
     from blockrank_amd import profiling, synthetic
     from transformers import MistralConfig, MistralModel
@@ -170,17 +174,28 @@ def bench_model(args):
     if not args.hf_layer_ops:
         br.patch_layer_ops(model)        # one-pass RMSNorm and SiLU-gate kernels instead of the model file's eager expressions
         br.patch_qkv(model)              # one GEMM for the Q, K and V projections of a layer
-    steps = args.steps if args.steps is not None else 10
-    warmup = args.warmup if args.warmup is not None else 2
     if args.padded:
         def forward(**kw):
             return ranker(ids, valid, pos, rows=rows, **kw)
+
+        def build_plan():
+            br.blockrank_attention_mask(batch_size=B, attention_mask=valid, dtype=torch.bfloat16).plan(32, 8)
     else:
         pk = br.pack_padded_batch(dict(input_ids=ids, position_ids=pos, attention_mask=valid))
         lens_dev = pk["block_lengths"]
 
         def forward(**kw):
             return ranker.forward_packed(pk["input_ids"], pk["position_ids"], lens_dev, rows, H=layout.H, **kw)
+
+        def build_plan():
+            br.BlockMask.from_lengths(lens_dev, H=layout.H, packed=True, dtype=torch.bfloat16).plan(32, 8)
+    # the request plan is built once per forward pass (inside the timed forward); its cost alone, second call
+    build_plan()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    build_plan()
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - t0) * 1e3
     for _ in range(warmup):
         scores = forward()
     torch.cuda.synchronize()
@@ -222,6 +237,7 @@ def bench_model(args):
                    "norm_and_gate": "model's eager expressions" if args.hf_layer_ops else "one-pass HIP kernels",
                    "qkv_projection": "three GEMMs" if args.hf_layer_ops else "one stacked GEMM"},
         "prefill_tok_per_s": layout.valid_tokens / (ms_per_step * 1e-3),
+        "plan_build_ms": plan_ms,
         "attention_ms_per_step": sum(kern_ms),
         "attention_share": sum(kern_ms) / ms_per_step,
         "dense_tflops": dense_flops / (ms_per_step * 1e-3) / 1e12,
@@ -232,7 +248,11 @@ def bench_model(args):
         "roofline_hbm": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "bytes_per_launch": alg_bytes},
     }
-    print(json.dumps(res))
+    return res
+
+
+def bench_model(args):
+    print(json.dumps(run_model(args, args.steps if args.steps is not None else 10, args.warmup if args.warmup is not None else 2)))
 
 
 def bench_backward(args, br, layout, wl, q, k, v, mask, scale):
@@ -292,6 +312,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="cfg2: leave out the end-to-end leg (the Mistral-7B-shaped ranking forward of --workload cfg3, five batches)")
     ap.add_argument("--graph", action="store_true", help="also time the step replayed from a HIP graph")
     ap.add_argument("--qk-fp8", action="store_true",
                     help="compute Q K^T in fp8 e4m3 (bf16 workloads with head dim 128; includes the quantisation pass)")
@@ -399,11 +421,15 @@ def main():
     alg_bytes = float(layout.valid_tokens) * D * esize * (2 * Nq + 2 * Nkv)
     tflops = flops / (kern_avg_ms * 1e-3) / 1e12
     gbs = alg_bytes / (kern_avg_ms * 1e-3) / 1e9
-    traffic = None
+    # HBM bytes per launch are not measured by this run: they come from the profiler's FETCH_SIZE / WRITE_SIZE counters,
+    # recorded with the command and the commit they were taken at
+    traffic, traffic_from = None, None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get(args.workload)
+            rec = json.load(open(tpath)).get(args.workload)
+            if rec:
+                traffic, traffic_from = rec["bytes_per_launch"], f"{rec['source']} (rocprofv3 counters, taken at commit {rec['commit']})"
         except Exception:
             traffic = None
 
@@ -431,7 +457,7 @@ def main():
         "kernel_us": {"prefill_avg": kern_avg_ms * 1e3, "prefill_p10": kern_ms[len(kern_ms) // 10] * 1e3,
                       "prefill_p50": kern_ms[len(kern_ms) // 2] * 1e3, "prefill_p90": kern_ms[(len(kern_ms) * 9) // 10] * 1e3},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tflops / PEAK_BF16_TFLOPS,
-                     "traffic": traffic, "kernel": "br_prefill_mfma_kernel", "flops_per_launch": flops},
+                     "traffic": traffic, "traffic_from": traffic_from, "kernel": "br_prefill_mfma_kernel", "flops_per_launch": flops},
         "roofline_hbm": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "bytes_per_launch": alg_bytes},
     }
@@ -440,6 +466,20 @@ def main():
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(layout, q, k, v, scale, dtype)
         res["cpu_baseline"]["gpu_over_cpu"] = res["value"] / res["cpu_baseline"]["value"]
+    if args.workload == "cfg2" and not args.no_e2e and not args.qk_fp8:
+        # the ranking request end to end: what the headline layer is one twenty-first of
+        del q, k, v, out, scores
+        torch.cuda.empty_cache()
+        m = run_model(args, steps=5, warmup=2)
+        res["e2e"] = {
+            "workload": m["config"]["workload"], "name": "cfg3", "requests_per_s": m["value"], "ms_per_batch": m["ms_per_step"],
+            "batch": m["config"]["batch"], "steps": 5, "warmup": 2, "prefill_tok_per_s": m["prefill_tok_per_s"],
+            "token_layout": m["config"]["token_layout"], "plan_build_ms": m["plan_build_ms"],
+            "attention_ms_per_batch": m["attention_ms_per_step"], "attention_share": m["attention_share"],
+            "attention_kernel_us_per_layer": m["kernel_us"]["prefill_avg"], "attention_launches": m["kernel_us"]["launches"],
+            "attention_roofline_frac_mfma": m["roofline"]["frac"], "attention_roofline_frac_hbm": m["roofline_hbm"]["frac"],
+            "dense_tflops": m["dense_tflops"],
+        }
     print(json.dumps(res))
 
 
