@@ -23,14 +23,17 @@ from .attention import (
     register_blockrank_attention,
     register_triton_blockrank_attention,
 )
-from .losses import compute_auxiliary_attention_loss, rank_documents
+from .losses import bracket_rows, compute_auxiliary_attention_loss, rank_documents
 from .ranker import TruncatedRanker
 from .collate import block_icr_collate_packed, pack_padded_batch
-from .rope import apply_rotary_pos_emb, patch_rotary, unpatch_rotary
+from .rope import apply_rotary_pos_emb, apply_rotary_pos_emb_fused, patch_rotary, rotate_k, rotate_q, unpatch_rotary
 from .layer_ops import patch_layer_ops, patch_qkv, rms_norm, silu_mul, unpatch_layer_ops, unpatch_qkv
 
 __all__ = [
     "apply_rotary_pos_emb",
+    "apply_rotary_pos_emb_fused",
+    "rotate_k",
+    "rotate_q",
     "patch_rotary",
     "unpatch_rotary",
     "rms_norm",
@@ -50,6 +53,7 @@ __all__ = [
     "register_blockrank_attention",
     "register_triton_blockrank_attention",
     "compute_auxiliary_attention_loss",
+    "bracket_rows",
     "rank_documents",
     "TruncatedRanker",
     "block_icr_collate_packed",

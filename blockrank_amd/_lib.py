@@ -20,6 +20,15 @@ BR_ERR_HIP = 3
 
 _I64x3 = c_int64 * 3
 
+
+class BrPrefillOptions(ctypes.Structure):
+    """struct BrPrefillOptions of include/blockrank_hip.h (same members, same order)."""
+    _fields_ = [("struct_bytes", c_size_t), ("ev_start", c_void_p), ("ev_stop", c_void_p), ("score_part", c_void_p),
+                ("score_part_bytes", c_size_t), ("score_rows", ctypes.c_int32), ("rank_R", ctypes.c_int32), ("fp8_tokens", c_int64),
+                ("lse", c_void_p), ("lse_strides", c_void_p), ("rope_cos", c_void_p), ("rope_sin", c_void_p),
+                ("rope_strides", c_void_p), ("rank_rows", c_void_p), ("rank_scores", c_void_p), ("rank_scale", c_float)]
+
+
 # name -> (restype, argtypes); the single place that mirrors include/blockrank_hip.h
 SIGNATURES = {
     "br_version": (c_int, []),
@@ -42,6 +51,8 @@ SIGNATURES = {
     "br_prefill_fwd_scores": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t,
                                       c_int, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),
+    "br_prefill_fwd_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                  c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t, c_void_p, c_void_p]),
     "br_prefill_fp8qk_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int64]),
     "br_prefill_fwd_fp8qk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_void_p, c_size_t,

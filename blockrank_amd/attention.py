@@ -289,6 +289,9 @@ def blockrank_attention(
     kernel_events=None,
     score_rows: int = 0,
     qk_fp8: bool = False,
+    q_rope=None,
+    rank_rows: Optional[torch.Tensor] = None,
+    rank_scale: float = 1.0,
 ):
     """Block-sparse prefill attention.  query (B, Nq, S, D), key/value (B, Nkv, S, D) with any
     (batch, head, token) strides; block_mask a BlockMask, a (B, M, H) bool tensor, or the reference's
@@ -305,7 +308,18 @@ def blockrank_attention(
     qk_fp8 (bf16 inputs, head dim 128): Q K^T of the prefix and document blocks is computed in fp8 e4m3
     (K with one power-of-two scale per (sequence, kv head), every query row with its own), P V
     stays bf16; the query block's rows, from which the scores are read, are computed in bf16 - the
-    reduced-precision variant for ranking (scores as accurate as the bf16 kernel's)."""
+    reduced-precision variant for ranking (scores as accurate as the bf16 kernel's).
+
+    q_rope=(cos, sin) (bf16, tables (B or 1, S, D) on query's token axis): ``query`` is the projection's output
+    without its rotary position embedding, and the kernel rotates every Q row when it loads it; ``key`` must come
+    rotated (``blockrank_amd.rope.rotate_k``).
+
+    rank_rows (B, R) with score_rows > 0: indices 0..score_rows-1 into the last score_rows positions of the query
+    block, known before the layer runs (the reference derives them from the labels, losses.py:43-48).  The
+    per-document scores of those rows - ``doc_scores_from_partials`` with out_scale = rank_scale - are then reduced
+    in the launch that merges the attention's split partials, and the call returns (out, partials, scores)."""
+    if rank_rows is not None and score_rows <= 0:
+        raise ValueError("rank_rows needs score_rows > 0")
     if isinstance(block_mask, torch.Tensor) and block_mask.dim() == 3:
         block_mask = BlockMask(block_mask, query.dtype)
     bm = _as_block_mask(block_mask)
@@ -323,8 +337,10 @@ def blockrank_attention(
     if query.dtype not in _DTYPE_CODE:
         raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
     assert key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value must share a dtype"
+    if q_rope is not None and (query.dtype != torch.bfloat16 or qk_fp8):
+        raise NotImplementedError("the rotary embedding inside the attention kernel takes bfloat16 inputs and not the fp8 variant")
     if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
-        if query.dtype != torch.bfloat16 or qk_fp8 or score_rows > 0:
+        if query.dtype != torch.bfloat16 or qk_fp8 or score_rows > 0 or q_rope is not None:
             # same contract as the reference's kernelised path (blockrank_triton_kernel_attention.py:759-761)
             raise NotImplementedError("Backward pass not implemented yet (bfloat16 attention without fused score partials has one)")
         return _AttentionWithGrad.apply(query, key, value, bm, float(scaling))
@@ -338,39 +354,49 @@ def blockrank_attention(
         plan = bm.plan(Nq, Nkv)
         out = torch.empty((Bt, S, Nq, D), dtype=query.dtype, device=dev)
         ws_bytes = lib.br_prefill_workspace_bytes(B, Nq, Nkv, D)
-        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         out_strides = _lib._I64x3(0 if packed else S * Nq * D, D, Nq * D)
-        ev0, ev1 = kernel_events if kernel_events is not None else (None, None)
+        opt = _lib.BrPrefillOptions()
+        opt.struct_bytes = _lib.ctypes.sizeof(opt)
+        if kernel_events is not None:
+            opt.ev_start, opt.ev_stop = kernel_events
+        keep = []                                     # what the option structure points to, alive until the call returns
         if qk_fp8:
             if query.dtype != torch.bfloat16 or D != 128:
                 raise NotImplementedError("the fp8 Q K^T variant takes bfloat16 inputs with head dim 128")
-            tokens = S if packed else B * S
-            f8_bytes = lib.br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, tokens)
-            ws8 = torch.empty(max(f8_bytes, 16), dtype=torch.uint8, device=dev)
-            part, sp_bytes = None, 0
-            if score_rows > 0:
-                sp_bytes = lib.br_score_partials_bytes(B, Nq, M, H, score_rows)
-                part = torch.empty(max(sp_bytes // 4, 4), dtype=torch.float32, device=dev)
-            _lib.check(lib.br_prefill_fwd_fp8qk(
-                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
-                _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed), out_strides, float(scaling),
-                tokens, ws8.data_ptr(), f8_bytes, score_rows, part.data_ptr() if part is not None else None, sp_bytes,
-                _stream_ptr(dev), ev0, ev1))
-            return (out, part) if score_rows > 0 else out
+            opt.fp8_tokens = S if packed else B * S
+            ws_bytes = lib.br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, opt.fp8_tokens)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        if q_rope is not None:
+            cos, sin = q_rope
+            assert cos.dim() == 3 and cos.shape == sin.shape and cos.shape[-2:] == (S, D) and cos.shape[0] in (1, Bt), \
+                "cos / sin must be (B or 1, S, D) on the token axis of query"
+            assert cos.dtype == query.dtype and sin.dtype == query.dtype and cos.is_cuda and sin.is_cuda
+            if cos.stride(-1) != 1 or cos.stride(0) % 8 or cos.stride(1) % 8 or cos.stride() != sin.stride():
+                cos, sin = cos.contiguous(), sin.contiguous()
+            cs = (_lib.c_int64 * 2)(0 if cos.shape[0] == 1 else cos.stride(0), cos.stride(1))
+            keep += [cos, sin, cs]
+            opt.rope_cos, opt.rope_sin = cos.data_ptr(), sin.data_ptr()
+            opt.rope_strides = _lib.ctypes.cast(cs, _lib.c_void_p)
+        part = scores = None
         if score_rows > 0:
-            sp_bytes = lib.br_score_partials_bytes(B, Nq, M, H, score_rows)
-            part = torch.empty(max(sp_bytes // 4, 4), dtype=torch.float32, device=dev)
-            _lib.check(lib.br_prefill_fwd_scores(
-                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
-                _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed), out_strides, float(scaling),
-                _DTYPE_CODE[query.dtype], ws.data_ptr(), ws_bytes, score_rows, part.data_ptr(), sp_bytes,
-                _stream_ptr(dev), ev0, ev1))
-            return out, part
-        _lib.check(lib.br_prefill_fwd_events(
+            opt.score_rows = score_rows
+            opt.score_part_bytes = lib.br_score_partials_bytes(B, Nq, M, H, score_rows)
+            part = torch.empty(max(opt.score_part_bytes // 4, 4), dtype=torch.float32, device=dev)
+            opt.score_part = part.data_ptr()
+        if rank_rows is not None:
+            assert rank_rows.shape[0] == B and rank_rows.dim() == 2, "rank_rows must be (B, R)"
+            rr = rank_rows.to(device=dev, dtype=torch.int32).contiguous()
+            scores = torch.empty((B, M - 2), dtype=torch.float32, device=dev)
+            keep.append(rr)
+            opt.rank_rows, opt.rank_R, opt.rank_scale, opt.rank_scores = rr.data_ptr(), rr.shape[1], float(rank_scale), scores.data_ptr()
+        _lib.check(lib.br_prefill_fwd_ex(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), plan.data_ptr(), B, Nq, Nkv, M, H, D,
             _lib.strides3(q, packed), _lib.strides3(k, packed), _lib.strides3(v, packed), out_strides, float(scaling),
-            _DTYPE_CODE[query.dtype], ws.data_ptr(), ws_bytes, _stream_ptr(dev), ev0, ev1))
-    return out
+            _DTYPE_CODE[query.dtype], ws.data_ptr(), ws_bytes, _lib.ctypes.byref(opt), _stream_ptr(dev)))
+        del keep
+    if rank_rows is not None:
+        return out, part, scores
+    return (out, part) if score_rows > 0 else out
 
 
 def fused_scores_supported(query: torch.Tensor, block_mask) -> bool:
@@ -415,10 +441,13 @@ class LastBlockScores:
     ``compute_auxiliary_attention_loss`` of this package accepts it directly; ``dense()`` produces the
     reference tensor for anything else."""
 
-    def __init__(self, query, key, block_mask: BlockMask, scaling: float, num_rows: int, scaled: bool = True, partials=None):
+    def __init__(self, query, key, block_mask: BlockMask, scaling: float, num_rows: int, scaled: bool = True, partials=None,
+                 ranked=None):
         self.query, self.key, self.block_mask = query, key, block_mask
         self.scaling, self.R, self.scaled = float(scaling), int(num_rows), scaled
         self.partials = partials if scaled else None    # per-tile (max, sum) pairs left by the attention kernel
+        # (rows, temperature, scores): per-document scores the attention call already reduced for these rows
+        self.ranked = ranked if scaled else None
         _, Nq, _, D = query.shape
         self.shape = torch.Size((block_mask.B, Nq, self.R, block_mask.M * block_mask.H))
         self.device, self.dtype = query.device, query.dtype
@@ -458,7 +487,11 @@ class LastBlockScores:
                           row_reduce: str = "mean", return_probs: bool = False):
         """Same for ``rows`` (B, R') given as indices 0..R-1 into the handle's own R rows (the last R
         positions of the query block).  Uses the partials the attention kernel left when there are
-        any; otherwise the stand-alone score kernels."""
+        any (or the scores themselves, when the attention call was told these very rows beforehand); otherwise the
+        stand-alone score kernels."""
+        if (self.ranked is not None and rows is self.ranked[0] and temperature == self.ranked[1] and head_reduce == "mean"
+                and row_reduce == "mean" and not return_probs):
+            return self.ranked[2]
         if self.partials is not None:
             return doc_scores_from_partials(self.partials, self.block_mask, rows, self.R, self.query.shape[1],
                                             self.key.shape[1], temperature=temperature, head_reduce=head_reduce,
@@ -617,6 +650,10 @@ def blockrank_attention_forward(
     ``materialize_scores=True`` or set BLOCKRANK_AMD_DENSE_SCORES=1 for the fp32 tensor itself, and
     ``unscaled_scores=True`` for the literal SDPA function's unscaled variant (:537, :643).
     ``qk_fp8=True`` (or BLOCKRANK_AMD_QK_FP8=1) computes Q K^T in fp8 e4m3 (see blockrank_attention).
+    ``score_rows_hint`` (B, R') int tensor with ``score_temperature`` (default 0.05): the rows (indices into the last
+    ``num_last_queries`` positions) the caller is going to ask the handle's ``doc_scores_window`` for with that
+    temperature and the default reductions; their scores are then reduced inside the attention call's second launch
+    and the handle returns them when asked with that same tensor object.
     """
     assert attention_mask is not None, "BlockRank attention requires an attention mask"
     bm = _as_block_mask(attention_mask)
@@ -649,14 +686,33 @@ def blockrank_attention_forward(
             and not _env_flag("BLOCKRANK_AMD_SEPARATE_SCORES"))
 
     qk_fp8 = bool(kwargs.get("qk_fp8", False)) or _env_flag("BLOCKRANK_AMD_QK_FP8")
+    # A query that came through rope.apply_rotary_pos_emb_fused is still unrotated and carries its cos / sin tables:
+    # the attention kernel rotates the rows it loads.  Where something else reads the query as well (the scoring
+    # layer's logits, the fp8 variant's quantiser, a backward pass), it is rotated here instead.
+    deferred = getattr(query, "_blockrank_rope", None)
+    q_rope = None
+    if deferred is not None:
+        if want or qk_fp8 or needs_grad or query.dtype != torch.bfloat16:
+            from .rope import rotate_q
+            query = rotate_q(query, deferred.cos, deferred.sin)
+        else:
+            q_rope = (deferred.cos, deferred.sin)
+    hint = kwargs.get("score_rows_hint", None) if fuse and bm.M >= 3 else None
+    temperature = float(kwargs.get("score_temperature", 0.05))
+    if hint is not None and not 1 <= hint.shape[-1] <= 16:
+        hint = None
     out = blockrank_attention(query, key, value, bm, scaling, kernel_events=kwargs.get("kernel_events", None),
-                              score_rows=R if fuse else 0, qk_fp8=qk_fp8)
-    partials = None
-    if fuse:
+                              score_rows=R if fuse else 0, qk_fp8=qk_fp8, q_rope=q_rope, rank_rows=hint,
+                              rank_scale=1.0 / (temperature * Nq * hint.shape[-1]) if hint is not None else 1.0)
+    partials = ranked = None
+    if hint is not None:
+        out, partials, scores = out
+        ranked = (hint, temperature, scores)
+    elif fuse:
         out, partials = out
     if not want:
         return out, None
-    handle = LastBlockScores(query, key, bm, scaling, R, scaled=scaled, partials=partials)
+    handle = LastBlockScores(query, key, bm, scaling, R, scaled=scaled, partials=partials, ranked=ranked)
     if needs_grad or kwargs.get("materialize_scores", False) or _env_flag("BLOCKRANK_AMD_DENSE_SCORES"):
         return out, handle.dense()
     return out, handle

@@ -7,18 +7,19 @@
 
 #include "../../include/blockrank_hip.h"
 #include "br_common.h"
+#include "br_score_tiles.h"
 
-void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int* plan,
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int* plan,
                     hipStream_t stream);
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                           hipEvent_t ev_start, hipEvent_t ev_stop);
+                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
 int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                            hipEvent_t ev_start, hipEvent_t ev_stop);
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
                          float* probs, const long long* sq, const long long* sk, int B, int Nq, int Nkv, int M, int H, int D,
                          int R, int T, float scale, float out_scale, int dtype, hipStream_t stream);
 int br_launch_prefill_fp8qk(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                            hipEvent_t ev_start, hipEvent_t ev_stop);
+                            hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
 void br_launch_quantize_fp8(const void* k, const int* plan, void* k8, unsigned* amax, float* scales, const long long* sk,
                             long long k8_b, long long k8_h, int B, int Nkv, int M, int H, int D, hipStream_t stream);
 int br_launch_rope(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
@@ -76,6 +77,9 @@ bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW) {
     *NW = nw;
     return true;
 }
+
+// Workgroups of the prefill kernel per compute unit (the launchers' choice: two of up to four waves, else one).
+int prefill_wgs_per_cu(int nw) { return nw <= 4 ? 2 : 1; }
 
 int n_compute_units() {
     static thread_local int cached_dev = -1, cached_cu = 0;
@@ -151,7 +155,11 @@ static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded
     if (plan_ints < need) return fail(BR_ERR_SPACE, "plan buffer holds %zu ints, %zu needed", plan_ints, need);
     if ((long long)br_plan_max_items(B, M, H, T) * g.NHG >= (1 << 24))
         return fail(BR_ERR_ARG, "batch too large for one plan (B=%d, M=%d, H=%d)", B, M, H);
-    br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, plan, static_cast<hipStream_t>(stream));
+    const int n_cu = n_compute_units();
+    if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
+    int par = n_cu * prefill_wgs_per_cu(nw) / g.NHG;       // workgroups of the prefill grid that share one head group's items
+    par = par < 1 ? 1 : par;
+    br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, par, plan, static_cast<hipStream_t>(stream));
     return check_launch("plan launch");
 }
 
@@ -192,15 +200,57 @@ size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int64_t t
     return up256(base) + up256((size_t)Nkv * tokens * D) + 2 * up256((size_t)B * Nkv * 4);
 }
 
-// fp8_tokens > 0: Q K^T in fp8 (inputs bf16, quantised into the workspace first); it is the length of the
-// token axis summed over the batch (B*M*H padded slots, or the packed token count).
+// Everything optional about a forward call, in one place (the entry points below fill in what they expose).
+struct PrefillExtras {
+    void* ev_start = nullptr;
+    void* ev_stop = nullptr;
+    int score_rows = 0;                  // with score_part: the query block's last rows whose score partials are left
+    float* score_part = nullptr;
+    size_t score_part_bytes = 0;
+    int64_t fp8_tokens = 0;              // > 0: Q K^T in fp8 (inputs bf16, K quantised into the workspace first); the length of
+                                         // the token axis summed over the batch (B*M*H padded slots, or the packed token count)
+    float* lse = nullptr;
+    const int64_t* lse_strides = nullptr;
+    const void* rope_cos = nullptr;
+    const void* rope_sin = nullptr;
+    const int64_t* rope_strides = nullptr;
+    const int32_t* rank_rows = nullptr;  // with rank_scores: per-document scores of these rows, reduced in the finish launch
+    int rank_R = 0;
+    float rank_scale = 1.f;
+    float* rank_scores = nullptr;
+};
+
+static PrefillExtras with_events(void* ev_start, void* ev_stop) {
+    PrefillExtras x;
+    x.ev_start = ev_start; x.ev_stop = ev_stop;
+    return x;
+}
+
 static int prefill_impl(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
                         int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                         const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
-                        void* stream, void* ev_start, void* ev_stop, int score_rows, float* score_part, size_t score_part_bytes,
-                        int64_t fp8_tokens = 0, float* lse = nullptr, const int64_t* lse_strides = nullptr) {
+                        void* stream, const PrefillExtras& x) {
+    void* const ev_start = x.ev_start;
+    void* const ev_stop = x.ev_stop;
+    const int score_rows = x.score_part ? x.score_rows : 0;
+    float* const score_part = x.score_part;
+    const size_t score_part_bytes = x.score_part_bytes;
+    const int64_t fp8_tokens = x.fp8_tokens;
+    float* const lse = x.lse;
+    const int64_t* const lse_strides = x.lse_strides;
+    const void* const rope_cos = x.rope_cos;
+    const void* const rope_sin = x.rope_sin;
+    const int64_t* const rope_strides = x.rope_strides;
     int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
     if (rc) return rc;
+    if (rope_cos || rope_sin) {
+        if (dtype != BR_DTYPE_BF16 || fp8_tokens > 0) return fail(BR_ERR_ARG, "the rotary embedding of Q inside the attention kernel needs the bf16 kernel");
+        if (!rope_cos || !rope_sin || !rope_strides) return fail(BR_ERR_ARG, "cos, sin and their strides must be given together");
+        if (!aligned16(rope_cos) || !aligned16(rope_sin)) return fail(BR_ERR_ARG, "cos and sin must be 16-byte aligned");
+        if (rope_strides[0] < 0 || rope_strides[1] < D || rope_strides[0] % 8 || rope_strides[1] % 8 || rope_strides[0] >= (int64_t(1) << 31) ||
+            rope_strides[1] >= (int64_t(1) << 31))
+            return fail(BR_ERR_ARG, "cos/sin strides (batch, token) must be multiples of 16 bytes below 2^31 elements, rows dense");
+    }
     if (lse && (dtype != BR_DTYPE_BF16 || fp8_tokens > 0 || !lse_strides)) return fail(BR_ERR_ARG, "the log-sum-exp output comes from the bf16 kernel only");
     if (score_part) {
         if (dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "score partials come from the bf16 kernel only; use br_doc_scores");
@@ -209,6 +259,12 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         if (!aligned16(score_part)) return fail(BR_ERR_ARG, "score_part must be 16-byte aligned");
         const size_t sneed = br_score_partials_bytes(B, Nq, M, H, score_rows);
         if (score_part_bytes < sneed) return fail(BR_ERR_SPACE, "score_part holds %zu bytes, %zu needed", score_part_bytes, sneed);
+    }
+    if (x.rank_rows || x.rank_scores) {
+        if (!x.rank_rows || !x.rank_scores) return fail(BR_ERR_ARG, "the rows to score and the scores output must be given together");
+        if (!score_part) return fail(BR_ERR_ARG, "per-document scores in the same call need the score partials buffer");
+        if (x.rank_R <= 0 || x.rank_R > 16) return fail(BR_ERR_ARG, "R=%d rows not supported (1..16)", x.rank_R);
+        if ((size_t)(M - 2) * sizeof(float) > 60 * 1024) return fail(BR_ERR_ARG, "too many documents (%d) for the score reduction", M - 2);
     }
     if (!q || !k || !v || !out || !plan) return fail(BR_ERR_ARG, "null pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(plan) || !aligned16(workspace))
@@ -248,6 +304,9 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     p.score_part = score_part;
     p.score_R = score_part ? score_rows : 0;
     p.qk_scales = nullptr;
+    p.rope_cos = rope_cos; p.rope_sin = rope_sin;
+    p.rope_b = rope_cos ? (unsigned)rope_strides[0] : 0u;
+    p.rope_t = rope_cos ? (unsigned)rope_strides[1] : 0u;
     p.k8 = nullptr;
     p.k8_b = p.k8_h = 0;
     p.lse = lse;
@@ -258,6 +317,14 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     if (combine_grid > 4 * n_cu) combine_grid = 4 * n_cu;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipEvent_t e0 = static_cast<hipEvent_t>(ev_start), e1 = static_cast<hipEvent_t>(ev_stop);
+    BrTileScoreParams rank = {};
+    const BrTileScoreParams* rankp = nullptr;
+    if (x.rank_scores) {
+        rank.part = score_part; rank.plan = plan; rank.rows = x.rank_rows; rank.scores = x.rank_scores; rank.probs = nullptr;
+        rank.B = B; rank.Nq = Nq; rank.M = M; rank.H = H; rank.R = x.rank_R; rank.Rw = score_rows;
+        rank.out_scale = x.rank_scale;
+        rankp = &rank;
+    }
     int lrc;
     if (fp8_tokens > 0) {
         const bool packed = k_strides[0] == 0;
@@ -276,9 +343,9 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         p.k8 = k8;
         p.k8_b = (unsigned)k8_b; p.k8_h = (unsigned)k8_h;
         p.qk_scales = scales;
-        lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1);
+        lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp);
     } else {
-        lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1)
+        lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
                                      : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s, e0, e1);
     }
     if (lrc) return fail(BR_ERR_ARG, "no kernel for head dim %d with %d query heads per kv head", D, g.G);
@@ -290,14 +357,14 @@ int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out
                           const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
                           void* stream, void* ev_start, void* ev_stop) {
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
-                        workspace, workspace_bytes, stream, ev_start, ev_stop, 0, nullptr, 0);
+                        workspace, workspace_bytes, stream, with_events(ev_start, ev_stop));
 }
 
 int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
                    int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                    const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
-                        workspace, workspace_bytes, stream, nullptr, nullptr, 0, nullptr, 0);
+                        workspace, workspace_bytes, stream, PrefillExtras());
 }
 
 size_t br_prefill_noalloc_max_workspace_bytes(void) { return BR_NOALLOC_SCRATCH_BYTES; }
@@ -332,7 +399,7 @@ int br_prefill_fwd_noalloc(const void* q, const void* k, const void* v, void* ou
     void* ws = nullptr;
     if ((rc = noalloc_scratch(&ws))) return rc;
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
-                        ws, need, stream, nullptr, nullptr, 0, nullptr, 0);
+                        ws, need, stream, PrefillExtras());
 }
 
 int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
@@ -341,8 +408,33 @@ int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out
                           int score_rows, float* score_part, size_t score_part_bytes, void* stream, void* ev_start,
                           void* ev_stop) {
     if (!score_part) return fail(BR_ERR_ARG, "score_part must be provided");
+    PrefillExtras x = with_events(ev_start, ev_stop);
+    x.score_rows = score_rows; x.score_part = score_part; x.score_part_bytes = score_part_bytes;
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
-                        workspace, workspace_bytes, stream, ev_start, ev_stop, score_rows, score_part, score_part_bytes);
+                        workspace, workspace_bytes, stream, x);
+}
+
+int br_prefill_fwd_ex(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                      int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                      const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
+                      const BrPrefillOptions* opt, void* stream) {
+    PrefillExtras x;
+    if (opt) {
+        if (opt->struct_bytes != sizeof(BrPrefillOptions))
+            return fail(BR_ERR_ARG, "BrPrefillOptions.struct_bytes is %zu, this library's structure has %zu", opt->struct_bytes, sizeof(BrPrefillOptions));
+        if (opt->fp8_tokens < 0) return fail(BR_ERR_ARG, "fp8_tokens must not be negative");
+        if ((opt->rope_cos || opt->rope_sin) && !(opt->rope_cos && opt->rope_sin && opt->rope_strides))
+            return fail(BR_ERR_ARG, "cos, sin and their strides must be given together");
+        if (opt->lse && (!opt->lse_strides || opt->lse_strides[0] < 0 || opt->lse_strides[1] <= 0)) return fail(BR_ERR_ARG, "bad lse strides");
+        x.ev_start = opt->ev_start; x.ev_stop = opt->ev_stop;
+        x.score_rows = opt->score_rows; x.score_part = opt->score_part; x.score_part_bytes = opt->score_part_bytes;
+        x.fp8_tokens = opt->fp8_tokens;
+        x.lse = opt->lse; x.lse_strides = opt->lse_strides;
+        x.rope_cos = opt->rope_cos; x.rope_sin = opt->rope_sin; x.rope_strides = opt->rope_strides;
+        x.rank_rows = opt->rank_rows; x.rank_R = opt->rank_R; x.rank_scale = opt->rank_scale; x.rank_scores = opt->rank_scores;
+    }
+    return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, dtype,
+                        workspace, workspace_bytes, stream, x);
 }
 
 int br_prefill_fwd_fp8qk(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
@@ -350,9 +442,11 @@ int br_prefill_fwd_fp8qk(const void* q, const void* k, const void* v, void* out,
                          const int64_t* out_strides, float scale, int64_t tokens, void* workspace, size_t workspace_bytes,
                          int score_rows, float* score_part, size_t score_part_bytes, void* stream, void* ev_start, void* ev_stop) {
     if (tokens <= 0) return fail(BR_ERR_ARG, "tokens must be positive (got %lld)", (long long)tokens);
+    PrefillExtras x = with_events(ev_start, ev_stop);
+    x.score_rows = score_rows; x.score_part = score_part; x.score_part_bytes = score_part_bytes;
+    x.fp8_tokens = tokens;
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale,
-                        BR_DTYPE_BF16, workspace, workspace_bytes, stream, ev_start, ev_stop, score_rows, score_part,
-                        score_part_bytes, tokens);
+                        BR_DTYPE_BF16, workspace, workspace_bytes, stream, x);
 }
 
 int br_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv, int M,
@@ -361,8 +455,10 @@ int br_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, c
                        const int64_t* lse_strides, void* stream) {
     if (!lse || !lse_strides) return fail(BR_ERR_ARG, "lse and its strides must be provided");
     if (lse_strides[0] < 0 || lse_strides[1] <= 0) return fail(BR_ERR_ARG, "bad lse strides");
+    PrefillExtras x;
+    x.lse = lse; x.lse_strides = lse_strides;
     return prefill_impl(q, k, v, out, plan, B, Nq, Nkv, M, H, D, q_strides, k_strides, v_strides, out_strides, scale, BR_DTYPE_BF16,
-                        workspace, workspace_bytes, stream, nullptr, nullptr, 0, nullptr, 0, 0, lse, lse_strides);
+                        workspace, workspace_bytes, stream, x);
 }
 
 size_t br_prefill_bwd_workspace_bytes(int B, int Nq, int Nkv, int H, int D, int64_t token_slots) {
@@ -498,8 +594,12 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
 int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
                int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* cs_strides, int dtype, void* stream) {
     if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "dtype must be fp32 (0) or bf16 (1)");
-    if (B <= 0 || Nq <= 0 || Nkv <= 0 || S <= 0) return fail(BR_ERR_ARG, "B, Nq, Nkv and S must be positive");
+    if (B <= 0 || Nq < 0 || Nkv <= 0 || S <= 0) return fail(BR_ERR_ARG, "B, Nkv and S must be positive, Nq not negative");
     if (D != 64 && D != 128) return fail(BR_ERR_ARG, "head dim %d not supported (64 or 128)", D);
+    const int64_t zero3[3] = {0, 0, 0};
+    if (Nq == 0) {       // K alone (Q is rotated by the attention kernel): the q arguments are not used
+        q = k; q_out = k_out; q_strides = zero3;
+    }
     if (!q || !k || !cos || !sin || !q_out || !k_out || !q_strides || !k_strides || !cs_strides) return fail(BR_ERR_ARG, "null pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(cos) || !aligned16(sin) || !aligned16(q_out) || !aligned16(k_out))
         return fail(BR_ERR_ARG, "q, k, cos, sin and the outputs must be 16-byte aligned");

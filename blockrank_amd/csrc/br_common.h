@@ -13,7 +13,9 @@
 #define BR_BN 64              // keys per key/value tile
 #define BR_RB 32              // query rows per wave (one 32x32 MFMA row block)
 #define BR_SLOTS_PER_SEQ 32   // split-KV partial slots available to one sequence's query block
+#ifndef BR_MIN_CHUNK
 #define BR_MIN_CHUNK 8        // a split of the query block's key walk covers at least this many tiles
+#endif
 
 // Plan buffer (int32):
 //   [header BR_PLAN_HDR][start B*M][len B*M][tok B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
@@ -256,6 +258,12 @@ struct BrPrefillParams {
     const float* qk_scales;
     const void* k8;
     unsigned k8_b, k8_h;
+    // Optional: rotary position embedding of Q applied by the attention kernel to the rows it loads (bf16 kernel
+    // only): cos and sin tables (batch or 1, tokens, D) on the same token axis as q, element strides rope_b (0: one
+    // table for the whole batch) and rope_t; q then holds the projection's output as it is.  Null: q is used as given.
+    const void* rope_cos;
+    const void* rope_sin;
+    unsigned rope_b, rope_t;
     // Optional: the log-sum-exp of every real query row, in base-2 units (log2 of the sum over the visible keys
     // of 2^(scale * log2(e) * q.k)), at lse[b * lse_b + head * lse_h + token]; the backward pass starts from it.
     // Null: not wanted.  Written by the streaming bf16 kernel and the finish kernel only.

@@ -69,15 +69,16 @@ __device__ int block_exclusive_scan(int x, int* sh, int* total) {
     return base + incl - x;
 }
 
-// Split count for query tile tt of the query block: enough splits that each covers about
-// BR_MIN_CHUNK key tiles, limited so that all tiles of the block fit the sequence's slot budget.
-__device__ inline int splits_for(int ntiles, int ns_cap) {
-    int ns = ceil_div(ntiles, BR_MIN_CHUNK);
+// Split count for a query tile of the query block: enough splits that each covers about ``chunk`` key tiles,
+// limited so that all tiles of the block fit the sequence's slot budget.
+__device__ inline int splits_for(int ntiles, int ns_cap, int chunk) {
+    int ns = ceil_div(ntiles, chunk);
     ns = ns < 1 ? 1 : ns;
     return ns > ns_cap ? ns_cap : ns;
 }
 
-__global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T, int packed) {
+// par: workgroups of the prefill grid per head group, i.e. how many of a plan's items run side by side.
+__global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T, int packed, int par) {
     __shared__ int sh[kPlanThreads / 64];
     __shared__ int s_bad;
     const int tid = threadIdx.x;
@@ -155,6 +156,29 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     if (tid < 8) s_qfirst[tid] = 0x7fffffff;
     __syncthreads();
 
+    // Length of a split of the query block's key walk.  The walk is cut so that the batch has enough items to fill
+    // the grid, and no further: every split costs a set-up, an epilogue and a set of partials to write and merge,
+    // while a split as long as the whole kernel's share per workgroup still ends with the others because the split
+    // items are handed out first.  So: about the estimated work per workgroup (all items' key tiles plus their
+    // constant, over the workgroups that run side by side), and at least BR_MIN_CHUNK.
+    long long w_all = 0;
+    for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
+        const int p = p0 + tid;
+        int w = 0;
+        if (p < BM) {
+            const int b = p / M, m = p - b * M;
+            const int L = len[p];
+            const int nq = ceil_div(L, T);
+            const int np = m == M - 1 ? (M > 1 ? prev_tiles[b] : 0) : (br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0);
+            for (int tt = 0; tt < nq; ++tt) w += item_weight(np, tt, L);
+        }
+        int tot;
+        block_exclusive_scan(w, sh, &tot);
+        w_all += tot;
+    }
+    int chunk = (int)(w_all / (par > 0 ? par : 1));
+    chunk = chunk < BR_MIN_CHUNK ? BR_MIN_CHUNK : chunk;
+
     struct Counts {
         int glob, x, w, comb;
     };
@@ -173,7 +197,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             ns_cap = ns_cap < 1 ? 1 : ns_cap;
             for (int tt = 0; tt < nq; ++tt) {
                 int e = (tt + 1) * T < L ? (tt + 1) * T : L;
-                int ns = splits_for(pt + ceil_div(e, BR_BN), ns_cap);
+                int ns = splits_for(pt + ceil_div(e, BR_BN), ns_cap, chunk);
                 c.glob += ns;
                 c.comb += ns > 1;
             }
@@ -253,7 +277,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                     int e = (tt + 1) * T < L ? (tt + 1) * T : L;
                     int nself = ceil_div(e, BR_BN);
                     int nt = pt + nself;
-                    int ns = splits_for(nt, ns_cap);
+                    int ns = splits_for(nt, ns_cap, chunk);
                     if (ns > 1) {
                         BrComb cb;
                         cb.b = b; cb.t0 = tt * T; cb.slot0 = slot; cb.nsplit = ns;
@@ -308,7 +332,7 @@ __global__ void br_block_table_from_len_kernel(const int* __restrict__ lens, int
 
 }  // namespace
 
-void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int* plan,
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int* plan,
                     hipStream_t stream) {
     int* start = plan + br_plan_off_start();
     int* len = plan + br_plan_off_len(B, M);
@@ -321,5 +345,5 @@ void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int 
         hipLaunchKernelGGL(br_block_table_from_len_kernel, dim3((BM + 255) / 256), dim3(256), 0, stream, lens, BM, H,
                            left_padded, start, len);
     }
-    hipLaunchKernelGGL(br_plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, plan, B, M, H, T, packed);
+    hipLaunchKernelGGL(br_plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, plan, B, M, H, T, packed, par);
 }

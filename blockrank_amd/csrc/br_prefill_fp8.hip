@@ -106,12 +106,14 @@ void br_launch_quantize_fp8(const void* k, const int* plan, void* k8, unsigned* 
 }
 
 // The prefill kernel with fp8 logits (p.k8: the quantised K, p.qk_scales: its scales) followed by
-// the split merge.  Returns 0 on success, -1 if (D, NW) has no instantiation (only D = 128 is built).
+// the split merge (with the score reduction ``rank`` asks for, if any).  Returns 0 on success, -1 if (D, NW) has no
+// instantiation (only D = 128 is built), 1 if the score reduction does not fit; nothing is launched then.
 int br_launch_prefill_fp8qk(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                            hipEvent_t ev_start, hipEvent_t ev_stop) {
+                            hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank) {
     const int per_cu = NW <= 4 ? 2 : 1;
     const int grid = n_cu * per_cu;
-    if (D != 128) return -1;
+    if (D != 128 || NW < 4 || NW > 8) return -1;
+    if (rank && (size_t)(rank->M - 2) * sizeof(float) > 60 * 1024) return 1;
     if (ev_start) (void)hipEventRecord(ev_start, stream);
     switch (NW) {
         case 4: launch8<128, 4>(p, grid, stream); break;
@@ -122,6 +124,5 @@ int br_launch_prefill_fp8qk(const BrPrefillParams& p, int D, int NW, int n_cu, i
         default: return -1;
     }
     if (ev_stop) (void)hipEventRecord(ev_stop, stream);
-    hipLaunchKernelGGL((br_finish_kernel<128>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
-    return 0;
+    return br_launch_finish<128>(p, NW, combine_grid, rank, stream);
 }

@@ -10,11 +10,13 @@ void launch(const BrPrefillParams& p, int grid, hipStream_t stream) {
 
 }  // namespace
 
-// Returns 0 on success, -1 if (D, NW) has no instantiation.
+// Returns 0 on success, -1 if (D, NW) has no instantiation, 1 if the score reduction asked for with ``rank`` does not
+// fit (nothing is launched in either case).
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                           hipEvent_t ev_start, hipEvent_t ev_stop) {
+                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank) {
     const int per_cu = NW <= 4 ? 2 : 1;
     const int grid = n_cu * per_cu;
+    if (rank && (size_t)(rank->M - 2) * sizeof(float) > 60 * 1024) return 1;
     if (ev_start) (void)hipEventRecord(ev_start, stream);
 #define BR_CASE(DD, WW)                                   \
     if (D == DD && NW == WW) {                            \
@@ -27,9 +29,5 @@ int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, in
     return -1;
 launched:
     if (ev_stop) (void)hipEventRecord(ev_stop, stream);
-    if (D == 128)
-        hipLaunchKernelGGL((br_finish_kernel<128>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
-    else
-        hipLaunchKernelGGL((br_finish_kernel<64>), dim3(combine_grid), dim3(256), 0, stream, p, NW);
-    return 0;
+    return D == 128 ? br_launch_finish<128>(p, NW, combine_grid, rank, stream) : br_launch_finish<64>(p, NW, combine_grid, rank, stream);
 }

@@ -31,6 +31,7 @@
 //   V    row = key; chunk c of row r sits at chunk c ^ ((r & 3) << 1).
 #pragma once
 #include "br_common.h"
+#include "br_score_tiles.h"
 
 namespace {
 
@@ -586,6 +587,10 @@ struct Prefill {
         // the rest of the set-up runs under their latency.
         Frag qf[D / 16];
         u32x4 qraw[F8 ? D / 16 : 1];       // fp8: the bf16 rows as loaded, converted once they have arrived
+        // rotary embedding applied here: the row's cos / sin values for the lane's dims (both halves of the tables)
+        constexpr int NRC = F8 ? 1 : D / 32;
+        bf16x8 rcos[2][NRC], rsin[2][NRC];
+        const bool rope = !F8 && p.rope_cos != nullptr && rb_active;
         {
             const char* qrow = reinterpret_cast<const char*>(p.q) +
                                ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)head +
@@ -605,6 +610,20 @@ struct Prefill {
                 for (int c = 0; c < D / 16; ++c) {
                     if constexpr (F8) qraw[c] = u32x4{0u, 0u, 0u, 0u};
                     else qf[c] = as_bf16x8(uint4{0u, 0u, 0u, 0u});
+                }
+            }
+            if constexpr (!F8) {
+                if (rope) {
+                    const long long tbl = ((long long)p.rope_b * b + (long long)p.rope_t * (qtok0 + row0 + (ln < last ? ln : last))) * 2 + lh * 16;
+                    const char* crow = reinterpret_cast<const char*>(p.rope_cos) + tbl;
+                    const char* srow = reinterpret_cast<const char*>(p.rope_sin) + tbl;
+#pragma unroll
+                    for (int c = 0; c < NRC; ++c) {
+                        rcos[0][c] = as_bf16x8(ld16(crow + c * 32));
+                        rcos[1][c] = as_bf16x8(ld16(crow + (c + NRC) * 32));
+                        rsin[0][c] = as_bf16x8(ld16(srow + c * 32));
+                        rsin[1][c] = as_bf16x8(ld16(srow + (c + NRC) * 32));
+                    }
                 }
             }
         }
@@ -668,6 +687,26 @@ struct Prefill {
             sc2 *= q_scale;
 #pragma unroll
             for (int c = 0; c < D / 16; ++c) qf[c] = quantize_q8(qraw[c], q_inv);
+        }
+        if constexpr (!F8) {
+            // out = x cos + rotate_half(x) sin: dim d < D/2 pairs with d + D/2, which the same lane holds D/32 chunks
+            // further on; fp32 arithmetic, one rounding (what the stand-alone rotary kernel computes)
+            if (rope) {
+#pragma unroll
+                for (int c = 0; c < NRC; ++c) {
+                    bf16x8 lo = qf[c], hi = qf[c + NRC];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float x1 = (float)lo[j], x2 = (float)hi[j];
+                        const float o1 = x1 * (float)rcos[0][c][j] - x2 * (float)rsin[0][c][j];
+                        const float o2 = x2 * (float)rcos[1][c][j] + x1 * (float)rsin[1][c][j];
+                        lo[j] = (__bf16)o1;
+                        hi[j] = (__bf16)o2;
+                    }
+                    qf[c] = lo;
+                    qf[c + NRC] = hi;
+                }
+            }
         }
 #pragma unroll
         for (int c = 0; c < D / 16; ++c) asm volatile("" : "+v"(qf[c]));
@@ -878,33 +917,47 @@ __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillPa
 // Finish: (1) merge the split-KV partials of the query block,
 // out = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m); one workgroup per (query tile, head group, row
 // block); (2) set the rows of padded token slots to zero.
-template <int D>
-__global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int NW) {
+// THREADS: workgroup size.  PATH >= 0 (with score_wgs > 0): the first score_wgs workgroups (one per sequence) turn
+// the score partials the prefill kernel left into per-document scores instead (sp, reduction PATH of
+// br_doc_final_tiles_body with sp_waves accumulator rows of LDS), the others share the merge as if they were the
+// whole grid.  PATH < 0: the merge alone.
+template <int D, int THREADS, int PATH>
+__global__ __launch_bounds__(THREADS) void br_finish_kernel(BrPrefillParams p, int NW, BrTileScoreParams sp, int score_wgs, int sp_waves) {
+    if constexpr (PATH >= 0) {
+        extern __shared__ float br_finish_dyn[];
+        if ((int)blockIdx.x < score_wgs) {
+            br_doc_final_tiles_body<PATH>(sp, blockIdx.x, br_finish_dyn, sp_waves);
+            return;
+        }
+    } else {
+        score_wgs = 0;
+    }
+    const int bid = blockIdx.x - score_wgs, nblk = gridDim.x - score_wgs;
     const BrGeom& ge = p.geom;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, ge.tpb * BR_RB);
     constexpr int CPR = D / 4;                    // float4 chunks per row = threads per row
-    constexpr int RPW = 256 / CPR;                // rows one workgroup merges at a time
-    constexpr int SUBS = BR_RB / RPW;             // such row groups per 32-row block
-    const int n_units = pv.hdr[BR_PH_NCOMB] * ge.NHG * NW * SUBS;
+    constexpr int RPW = THREADS / CPR;            // rows one workgroup merges at a time
+    const int rows = NW * BR_RB;                  // rows of one (combine entry, head group): NW query-tile waves of 32
+    const int subs = (rows + RPW - 1) / RPW;      // such row groups
+    const int n_units = pv.hdr[BR_PH_NCOMB] * ge.NHG * subs;
     const BrComb* combs = pv.comb;
     const int m = p.M - 1;
-    const int rows = NW * BR_RB;
     const int rr = threadIdx.x / CPR, cc = threadIdx.x % CPR;
-    for (int u = blockIdx.x; u < n_units; u += gridDim.x) {
-        const int subu = u % SUBS;
-        const int wave = (u / SUBS) % NW;
-        const int w = u / (SUBS * NW);
+    for (int u = bid; u < n_units; u += nblk) {
+        const int subu = u % subs;
+        const int w = u / subs;
         const int ci = w / ge.NHG, hg = w - ci * ge.NHG;
+        const int r = subu * RPW + rr;                               // row inside the slot
+        if (r >= rows) continue;
+        const int wave = r / BR_RB, rloc = r - wave * BR_RB;         // the prefill wave that owned it, row of its 32
         const BrComb c = combs[ci];
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int len_m = pv.len[c.b * p.M + m];
         const int qtok0 = pv.tok[c.b * p.M + m];
         const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
-        const int rloc = subu * RPW + rr;                            // row inside the 32-row block
         const int row = c.t0 + sub * BR_RB + rloc;
         if (row >= len_m) continue;
         const int head = kvh * ge.G + hsub * ge.Gw + g;
-        const int r = wave * BR_RB + rloc;
         const long long slot0 = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0) * ge.NHG + hg;
         const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
         const float2* ml = reinterpret_cast<const float2*>(p.part_ml) + slot0 * rows + r;
@@ -946,8 +999,12 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
     // Padded token slots: no kernel computes them, so give them a defined value (zero).  The prefill kernel
     // does that for the documents it has items for; what is left here are the prefix, the query block and
     // documents with no real token at all (a packed layout has no padded slots).
+    // One (block, head) per wave and step: the loop is a chain of dependent loads (block table, then the stores'
+    // addresses), so what counts is how many of them are in flight.
     const int n_pad_work = pv.hdr[BR_PH_PACKED] ? 0 : p.B * p.M * p.Nq;
-    for (int w = blockIdx.x; w < n_pad_work; w += gridDim.x) {
+    constexpr int WAVES = THREADS / 64;
+    const int lane = threadIdx.x & 63;
+    for (int w = bid * WAVES + (threadIdx.x >> 6); w < n_pad_work; w += nblk * WAVES) {
         const int bm = w / p.Nq, head = w - bm * p.Nq;
         const int b = bm / p.M, mm = bm - b * p.M;
         const int st = pv.start[bm], ln = pv.len[bm];
@@ -955,13 +1012,39 @@ __global__ __launch_bounds__(256) void br_finish_kernel(BrPrefillParams p, int N
         const int npad = p.H - ln;
         constexpr int CP8 = D / 8;
         __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
-        for (int idx = threadIdx.x; idx < npad * CP8; idx += blockDim.x) {
+        for (int idx = lane; idx < npad * CP8; idx += 64) {
             int r = idx / CP8, c8 = idx - r * CP8;
             int pos = r < st ? r : r + ln;
             uint4 z = {0u, 0u, 0u, 0u};
             *reinterpret_cast<uint4*>(obase + (long long)(mm * p.H + pos) * p.so_t + c8 * 8) = z;
         }
     }
+}
+
+// Launch of the finish kernel after a prefill kernel.  sp: the per-document score reduction to run in the same
+// launch (its partials are those the prefill kernel just wrote), or nullptr.  Returns 1 when the reduction's
+// accumulator rows do not fit the LDS (too many documents), with nothing launched.
+template <int D>
+inline int br_launch_finish(const BrPrefillParams& p, int NW, int combine_grid, const BrTileScoreParams* sp, hipStream_t stream) {
+    BrTileScoreParams none = {};
+    if (!sp) {
+        hipLaunchKernelGGL((br_finish_kernel<D, 256, -1>), dim3(combine_grid), dim3(256), 0, stream, p, NW, none, 0, 0);
+        return 0;
+    }
+    const int docs = sp->M - 2;
+    const int path = br_doc_final_path(docs, sp->H);
+    int nwaves = path == 0 ? 16 : 8;
+    while (nwaves > 1 && (size_t)nwaves * docs * sizeof(float) > 48 * 1024) nwaves >>= 1;
+    const size_t lds = (size_t)nwaves * docs * sizeof(float);
+    if (lds > 60 * 1024) return 1;
+    const int grid = sp->B + (path == 0 ? (combine_grid + 3) / 4 : (combine_grid + 1) / 2);
+    if (path == 0)
+        hipLaunchKernelGGL((br_finish_kernel<D, 1024, 0>), dim3(grid), dim3(1024), lds, stream, p, NW, *sp, sp->B, nwaves);
+    else if (path == 1)
+        hipLaunchKernelGGL((br_finish_kernel<D, 512, 1>), dim3(grid), dim3(512), lds, stream, p, NW, *sp, sp->B, nwaves);
+    else
+        hipLaunchKernelGGL((br_finish_kernel<D, 512, 2>), dim3(grid), dim3(512), lds, stream, p, NW, *sp, sp->B, nwaves);
+    return 0;
 }
 
 }  // namespace

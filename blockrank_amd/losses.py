@@ -45,18 +45,21 @@ def compute_auxiliary_attention_loss(
     answer_ids: torch.Tensor | None = None,
     temperature: float = 0.05,
     return_logits=False,
+    rows: torch.Tensor | None = None,
 ):
     """(B, M-2) per-document logits (and, with ``answer_ids``, the InfoNCE loss and accuracy).
 
     attention_scores: LastBlockScores handle or (B, N, h1, M*H) tensor; labels (B, M*H) with -100 on
     everything but the completion; attention_mask (B, M, H).  Follows losses.py:37-78: rows =
     {bracket-1, bracket}; softmax over all document tokens jointly; sum per document; mean over heads
-    and the two rows; divide by temperature.
+    and the two rows; divide by temperature.  ``rows``: the result of ``bracket_rows(labels, h1)`` if the caller
+    already has it (the tensor given to the model call as ``score_rows_hint``: the handle then holds the scores).
     """
     B, M, H = attention_mask.shape
     _, N, h1, MH = attention_scores.shape
     assert MH == M * H, "Attention scores last dimension must match M*H"
-    rows = bracket_rows(labels, h1)                                  # (B, 2) in [0, h1)
+    if rows is None:
+        rows = bracket_rows(labels, h1)                              # (B, 2) in [0, h1)
     if isinstance(attention_scores, LastBlockScores) and attention_scores.needs_grad():
         attention_scores = attention_scores.dense()          # training: the differentiable logits tensor
     if isinstance(attention_scores, LastBlockScores):

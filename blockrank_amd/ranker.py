@@ -33,6 +33,16 @@ def _decoder(model):
     return base
 
 
+def _module_rotary(attn):
+    """The rotary function of the file the attention class lives in - unless it is this package's variant that leaves
+    Q to the attention kernel: the scoring layer's queries go to the score kernels, which take them rotated."""
+    fn = sys.modules[type(attn).__module__].apply_rotary_pos_emb
+    if getattr(fn, "_blockrank_fused_q", False):
+        from .rope import apply_rotary_pos_emb
+        return apply_rotary_pos_emb
+    return fn
+
+
 class TruncatedRanker:
     """scores = TruncatedRanker(model, layer_idx)(input_ids, attention_mask, position_ids, labels)
 
@@ -84,7 +94,7 @@ class TruncatedRanker:
         # the scoring layer: keys of all tokens, queries of the query block only
         layer = base.layers[self.layer_idx]
         attn = layer.self_attn
-        rope = sys.modules[type(attn).__module__].apply_rotary_pos_emb
+        rope = _module_rotary(attn)
         D = attn.head_dim
         x = layer.input_layernorm(hidden)
         k = attn.k_proj(x).view(B, S, -1, D).transpose(1, 2)           # (B, Nkv, S, D)
@@ -125,7 +135,7 @@ class TruncatedRanker:
                 hidden = hidden[0]
         layer = base.layers[self.layer_idx]
         attn = layer.self_attn
-        rope = sys.modules[type(attn).__module__].apply_rotary_pos_emb
+        rope = _module_rotary(attn)
         D = attn.head_dim
         for name in ("q_norm", "k_norm"):
             if hasattr(attn, name):

@@ -51,7 +51,54 @@ def apply_rotary_pos_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, si
     return _rotate(q, k, cos, sin, unsqueeze_dim)
 
 
-def _rotate(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqueeze_dim: int = 1):
+class DeferredRotary:
+    """What ``apply_rotary_pos_emb_fused`` leaves on the query tensor: the tables the attention kernel rotates its
+    Q rows with."""
+
+    def __init__(self, cos: torch.Tensor, sin: torch.Tensor):
+        self.cos, self.sin = cos, sin
+
+
+def rotate_k(k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """The rotary embedding of K alone (same kernel, no query heads): (B, Nkv, S, D) in, the same logical shape out,
+    stored as (B, S, Nkv, D)."""
+    return _rotate(None, k, cos, sin)[1]
+
+
+def rotate_q(q: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """The rotary embedding of a query tensor alone (the kernel takes a key tensor along: its first head goes twice)."""
+    return _rotate_impl(q, q[:, :1], cos, sin)[0]
+
+
+def apply_rotary_pos_emb_fused(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqueeze_dim: int = 1):
+    """Signature of the model files' ``apply_rotary_pos_emb``; K is rotated here, Q is returned as it came with the
+    tables attached (``q._blockrank_rope``): the BlockRank attention hook of this package hands them to the attention
+    kernel, which rotates every Q row in registers when it loads it - two passes over the largest tensor of the layer
+    less.  Only for inference through that hook (bf16): any other consumer of the returned q would see it unrotated, so
+    with gradients enabled, or dtypes the fused path does not take, both tensors are rotated here as usual."""
+    fused_ok = (q.dtype == torch.bfloat16 and q.is_cuda and cos.dim() == 3
+                and not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad)))
+    if not fused_ok:
+        return apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim)
+    assert unsqueeze_dim == 1, "only the (batch, heads, tokens, dim) convention of the decoder layers is supported"
+    k_out = rotate_k(k, cos, sin)
+    q._blockrank_rope = DeferredRotary(cos, sin)
+    return q, k_out
+
+
+apply_rotary_pos_emb_fused._blockrank_fused_q = True
+
+
+def _rotate(q, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqueeze_dim: int = 1):
+    if q is None:                      # K alone
+        return None, _rotate_impl(None, k, cos, sin)[1]
+    return _rotate_impl(q, k, cos, sin, unsqueeze_dim)
+
+
+def _rotate_impl(q, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqueeze_dim: int = 1):
+    k_only = q is None
+    if k_only:
+        q = k
     assert unsqueeze_dim == 1, "only the (batch, heads, tokens, dim) convention of the decoder layers is supported"
     assert q.is_cuda and k.is_cuda and cos.is_cuda and sin.is_cuda, "the rotary embedding kernel needs device tensors"
     assert q.dtype == k.dtype == cos.dtype == sin.dtype and q.dtype in _DTYPE_CODE, "q, k, cos and sin must share a dtype (bf16 or fp32)"
@@ -66,17 +113,24 @@ def _rotate(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tens
     if cos.stride(-1) != 1 or cos.stride(0) % per16 or cos.stride(1) % per16 or cos.stride() != sin.stride():
         cos, sin = cos.contiguous(), sin.contiguous()
     with torch.cuda.device(q.device):
-        q_out = torch.empty((B, S, Nq, D), dtype=q.dtype, device=q.device)
         k_out = torch.empty((B, S, Nkv, D), dtype=q.dtype, device=q.device)
         cs = _I64x2(0 if cos.shape[0] == 1 else cos.stride(0), cos.stride(1))
+        if k_only:
+            _lib.check(lib.br_rope_qk(None, k.data_ptr(), cos.data_ptr(), sin.data_ptr(), None, k_out.data_ptr(), B, 0, Nkv,
+                                      S, D, None, _lib.strides3(k), cs, _DTYPE_CODE[q.dtype], _stream_ptr(q.device)))
+            return None, k_out.transpose(1, 2)
+        q_out = torch.empty((B, S, Nq, D), dtype=q.dtype, device=q.device)
         _lib.check(lib.br_rope_qk(q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(), q_out.data_ptr(), k_out.data_ptr(), B, Nq, Nkv,
                                   S, D, _lib.strides3(q), _lib.strides3(k), cs, _DTYPE_CODE[q.dtype], _stream_ptr(q.device)))
     return q_out.transpose(1, 2), k_out.transpose(1, 2)
 
 
-def patch_rotary(model) -> list[str]:
+def patch_rotary(model, fuse_q: bool = False) -> list[str]:
     """Replace ``apply_rotary_pos_emb`` in the module(s) that define the attention classes of ``model`` (a
-    Hugging Face decoder).  Returns the names of the patched modules; ``unpatch_rotary`` restores them."""
+    Hugging Face decoder).  Returns the names of the patched modules; ``unpatch_rotary`` restores them.
+    ``fuse_q=True`` installs ``apply_rotary_pos_emb_fused`` instead: K is rotated by the kernel here, Q by the
+    attention kernel (the model's attention implementation must be one of this package's BlockRank names)."""
+    fn = apply_rotary_pos_emb_fused if fuse_q else apply_rotary_pos_emb
     done = []
     for m in model.modules():
         mod = sys.modules.get(type(m).__module__)
@@ -84,7 +138,7 @@ def patch_rotary(model) -> list[str]:
             continue
         if getattr(mod.apply_rotary_pos_emb, "__module__", "") != __name__:
             mod._blockrank_amd_saved_rotary = mod.apply_rotary_pos_emb
-            mod.apply_rotary_pos_emb = apply_rotary_pos_emb
+        mod.apply_rotary_pos_emb = fn
         done.append(mod.__name__)
     return done
 

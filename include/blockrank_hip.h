@@ -128,6 +128,58 @@ int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out
                           void* workspace, size_t workspace_bytes, int score_rows, float* score_part,
                           size_t score_part_bytes, void* stream, void* ev_start, void* ev_stop);
 
+/* Everything optional about a forward call in one structure, for br_prefill_fwd_ex.  Zero-initialise it, set
+ * struct_bytes = sizeof(BrPrefillOptions) and fill in what the call should do; members left zero / NULL switch
+ * their feature off.
+ *   ev_start, ev_stop   hipEvent_t recorded around the main kernel, as in br_prefill_fwd_events.
+ *   score_part, score_part_bytes, score_rows
+ *                       the score partials of br_prefill_fwd_scores (bf16).
+ *   fp8_tokens          > 0: the fp8 Q K^T variant of br_prefill_fwd_fp8qk; the workspace is then sized by
+ *                       br_prefill_fp8qk_workspace_bytes.
+ *   lse, lse_strides    the log-sum-exp output of br_prefill_fwd_lse (bf16, no fp8).
+ *   rope_cos, rope_sin, rope_strides
+ *                       the rotary position embedding of Q inside the attention kernel (bf16, no fp8): q holds the
+ *                       query projection's output as it is, cos and sin are the tables (batch or 1, tokens, D) of the
+ *                       model's rotary module on q's token axis (rope_strides: element strides of batch and token,
+ *                       multiples of 8; a batch stride of 0 is one table for all sequences), and every Q row is rotated
+ *                       in registers when the kernel loads it: x cos + rotate_half(x) sin in fp32, rounded once, as
+ *                       br_rope_qk computes it.  K must come rotated (br_rope_qk with Nq = 0 does K alone).  Replaces
+ *                       the Q half of apply_rotary_pos_emb in the Hugging Face model files (transformers
+ *                       models/mistral/modeling_mistral.py, the same in llama and qwen2), which the reference reaches
+ *                       through the model forward of scripts/eval_attn.py:139-151.
+ *   rank_rows, rank_R, rank_scale, rank_scores
+ *                       with score_part: the per-document scores of br_doc_scores_from_partials(score_part, plan,
+ *                       rank_rows, rank_R, score_rows, ..., out_scale = rank_scale, scores = rank_scores, probs = NULL)
+ *                       for a caller that knows the rows to score before the layer runs (the reference finds them
+ *                       from the labels, losses.py:43-48, which do not depend on the forward): the reduction runs in the
+ *                       first workgroups of the launch that merges the split partials, so the whole call is two launches.
+ *                       rank_rows (B, rank_R) int32 and rank_scores (B, M-2) fp32 on the device. */
+typedef struct BrPrefillOptions {
+    size_t struct_bytes;
+    void* ev_start;
+    void* ev_stop;
+    float* score_part;
+    size_t score_part_bytes;
+    int32_t score_rows;
+    int32_t rank_R;
+    int64_t fp8_tokens;
+    float* lse;
+    const int64_t* lse_strides;
+    const void* rope_cos;
+    const void* rope_sin;
+    const int64_t* rope_strides;
+    const int32_t* rank_rows;
+    float* rank_scores;
+    float rank_scale;
+} BrPrefillOptions;
+
+/* br_prefill_fwd with the options above (opt may be NULL: then it is br_prefill_fwd).  Same checks and error codes as
+ * the single-purpose entry points, which are this call with one feature set. */
+int br_prefill_fwd_ex(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
+                      int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                      const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
+                      const BrPrefillOptions* opt, void* stream);
+
 /* Bytes of scratch br_prefill_fwd_fp8qk needs: the split-KV partials plus the quantised K and its scales.
  * tokens: length of the token axis summed over the batch (B*M*H for the padded layout, the number of
  * real tokens for a packed one). */
@@ -198,6 +250,8 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
  *   cos, sin (B, S, D) with element strides (batch, token) - a batch stride of 0 broadcasts one table;
  *   q_out (B, S, Nq, D), k_out (B, S, Nkv, D) contiguous: the layout whose head-transposed views the
  *   attention entry points take.  dtype 0 fp32, 1 bf16 for all six tensors; D 64 or 128.
+ *   Nq = 0 rotates K alone (q, q_out and q_strides are then ignored and may be NULL): the step that goes with
+ *   the rope_cos / rope_sin option of br_prefill_fwd_ex, which rotates Q itself.
  * fp32 arithmetic with one rounding of the result (the reference's eager bf16 expression rounds every
  * intermediate product and the sum). */
 int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,

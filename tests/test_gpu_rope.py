@@ -146,3 +146,74 @@ def test_patched_model_trains_through_the_rotation():
     for n in ref:
         assert got[n].abs().max().item() > 0
         torch.testing.assert_close(got[n], ref[n], rtol=1e-3, atol=1e-5 * ref[n].abs().max().item() + 1e-7)
+
+
+@pytest.mark.parametrize("Nq,Nkv,D", [(8, 2, 128), (4, 4, 64), (14, 2, 128)])
+def test_attention_kernel_rotates_q_rows_itself(Nq, Nkv, D):
+    """blockrank_attention(..., q_rope=(cos, sin)) on the unrotated Q against the oracle's rotation followed by the
+    oracle's attention, and against the two-kernel path (stand-alone rotation, then attention): same result to a
+    bf16 rounding of a Q element here and there."""
+    from tests._util import max_abs_on_real_rows, oracle_attention, oracle_doc_scores, assert_scores_close
+    from blockrank_amd.rope import rotate_k
+    lay = synthetic.make_layout([[40, 100, 7, 160, 33, 20], [64, 0, 150, 90, 65, 31]])
+    q, k, v = synthetic.random_qkv(lay, Nq, Nkv, D, torch.bfloat16, DEV, seed=11)
+    g = torch.Generator().manual_seed(5)
+    ang = torch.rand(lay.B, lay.S, D // 2, generator=g) * 6.28
+    ang = torch.cat([ang, ang * 1.1], dim=-1)                          # halves that differ: nothing may rely on their equality
+    cos, sin = ang.cos().to(DEV, torch.bfloat16), ang.sin().to(DEV, torch.bfloat16)
+    mask = br.BlockMask(lay.valid.to(DEV), torch.bfloat16)
+    scale = D ** -0.5
+    k_rot = rotate_k(k, cos, sin)
+    out, part = br.blockrank_attention(q, k_rot, v, mask, scale, score_rows=16, q_rope=(cos, sin))
+    # oracle: rotation in float64, rounded to bf16 like the tensors the attention oracle is given elsewhere
+    c64, s64 = cos.double().cpu().numpy(), sin.double().cpu().numpy()
+    q_ref = torch.as_tensor(orc.rotary_embedding(q.double().cpu().numpy(), c64, s64)).to(torch.bfloat16)
+    k_ref = torch.as_tensor(orc.rotary_embedding(k.double().cpu().numpy(), c64, s64)).to(torch.bfloat16)
+    assert max_abs_on_real_rows(out, oracle_attention(q_ref, k_ref, v, lay, scale), lay) <= 2e-2
+    rows = torch.tensor([[14, 15]] * lay.B, dtype=torch.int32, device=DEV)
+    scores = br.doc_scores_from_partials(part, mask, rows, 16, Nq, Nkv)
+    assert_scores_close(scores, oracle_doc_scores(q_ref, k_ref, lay, scale), rel=2e-3)
+    q_rot, _ = br.apply_rotary_pos_emb(q, k, cos, sin)
+    two = br.blockrank_attention(q_rot, k_rot, v, mask, scale)
+    real = lay.valid.reshape(lay.B, lay.S).to(DEV)
+    assert (out[real].float() - two[real].float()).abs().max().item() <= 4e-3
+    # one table for the whole batch, and the packed layout
+    cos1, sin1 = cos[:1].contiguous(), sin[:1].contiguous()
+    k1 = rotate_k(k, cos1, sin1)
+    a = br.blockrank_attention(q, k1, v, mask, scale, q_rope=(cos1, sin1))
+    b = br.blockrank_attention(br.apply_rotary_pos_emb(q, k, cos1, sin1)[0], k1, v, mask, scale)
+    assert (a[real].float() - b[real].float()).abs().max().item() <= 4e-3
+    with pytest.raises(NotImplementedError):
+        br.blockrank_attention(q, k_rot, v, mask, scale, q_rope=(cos, sin), qk_fp8=True)
+
+
+@pytest.mark.parametrize("kind", ["mistral", "qwen2"])
+def test_model_with_q_rotation_left_to_the_attention_kernel(kind):
+    """patch_rotary(model, fuse_q=True): hidden states and ranking scores of a small model as with the model file's own
+    rotary function; a layer that returns scores, and a training step, rotate Q before the hook uses it."""
+    from tests.test_gpu_hf_model import build
+    br.register_blockrank_attention()
+    model = build(kind, torch.bfloat16)
+    model.set_attn_implementation("sdpa_blockrank")
+    lay = synthetic.make_layout([[12, 30, 17, 25, 9], [10, 22, 31, 8, 11]])
+    ids = torch.randint(0, 512, (lay.B, lay.S), generator=torch.Generator().manual_seed(1)).to(DEV)
+    pos, valid, labels = lay.position_ids.to(DEV), lay.valid.to(DEV), lay.labels.to(DEV)
+    ranker = br.TruncatedRanker(model, layer_idx=2)
+    rows = lay.valid.reshape(lay.B, lay.S).to(DEV)
+
+    def run():
+        with torch.no_grad():
+            o = model(input_ids=ids, position_ids=pos, attention_mask=valid, output_hidden_states=True, output_attentions=True,
+                      layers_to_return_scores=[1], use_cache=False)
+            s1 = br.compute_auxiliary_attention_loss(o.attentions[0], labels, valid, answer_ids=None, return_logits=True)
+            return o.hidden_states[-1], s1, ranker(ids, valid, pos, labels)
+
+    ref_h, ref_s1, ref_s = run()
+    br.patch_rotary(model, fuse_q=True)
+    try:
+        got_h, got_s1, got_s = run()
+    finally:
+        br.unpatch_rotary(model)
+    assert (got_h.float() - ref_h.float())[rows].abs().max().item() <= 6e-2
+    torch.testing.assert_close(got_s1, ref_s1, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got_s, ref_s, rtol=2e-2, atol=2e-2)

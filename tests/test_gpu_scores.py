@@ -11,6 +11,7 @@ from tests._util import assert_scores_close, eval_rows, oracle_doc_scores
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+R_MIN = 16
 
 
 def fused(q, k, lay, scale, rows=None, **kw):
@@ -173,3 +174,61 @@ def test_dropout_in_training_is_refused():
     Mod.training = False
     out, _ = br.blockrank_attention_forward(Mod(), q, k, v, mask, 0.125, dropout=0.1)      # evaluation: dropout is off anyway
     assert out.shape == (1, lay.S, 4, 64)
+
+
+@pytest.mark.parametrize("docs,H", [(20, 160), (100, 96), (300, 40)])
+@pytest.mark.parametrize("qk_fp8", [False, True])
+def test_scores_reduced_inside_the_attention_call(docs, H, qk_fp8):
+    """rank_rows: the per-document scores come out of the launch that merges the split partials - bit-identical to
+    the separate reduction of the same partials (one-document-per-lane, four-per-lane and general paths), the
+    attention output untouched; through the hook with score_rows_hint, and two calls in a row (LDS and partials of
+    the first must not leak into the second)."""
+    g = torch.Generator().manual_seed(docs)
+    lens = [[int(x) for x in torch.randint(1, H + 1, (docs + 2,), generator=g)] for _ in range(2)]
+    lens[1][3] = 0                                                    # an empty document
+    lens[0][-1] = H
+    lens[1][-1] = max(R_MIN, H - 3)
+    lay = synthetic.make_layout(lens, H=H)
+    Nq, Nkv, D = 8, 2, 128
+    q, k, v = synthetic.random_qkv(lay, Nq, Nkv, D, torch.bfloat16, DEV, seed=3)
+    mask = br.BlockMask(lay.valid.to(DEV), torch.bfloat16)
+    scale = D ** -0.5
+    R = min(16, H)
+    rows = torch.tensor([[R - 2, R - 1], [R - 5, R - 1]], dtype=torch.int32, device=DEV)
+    out_scale = 1.0 / (0.05 * Nq * 2)
+    out0, part0 = br.blockrank_attention(q, k, v, mask, scale, score_rows=R, qk_fp8=qk_fp8)
+    want = br.doc_scores_from_partials(part0, mask, rows, R, Nq, Nkv)
+    for _ in range(2):
+        out1, part1, got = br.blockrank_attention(q, k, v, mask, scale, score_rows=R, qk_fp8=qk_fp8, rank_rows=rows, rank_scale=out_scale)
+        assert torch.equal(got, want)
+        assert torch.equal(out1, out0)                       # (the partials buffer has slots no kernel writes: not compared)
+
+    class Layer:
+        layer_idx = 3
+        num_key_value_groups = Nq // Nkv
+        training = False
+    out2, handle = br.blockrank_attention_forward(Layer(), q, k, v, mask, scale, layers_to_return_scores=[3], score_rows_hint=rows,
+                                                   qk_fp8=qk_fp8)
+    assert torch.equal(out2, out0)
+    assert handle.ranked is not None and handle.doc_scores_window(rows, temperature=0.05) is handle.ranked[2]
+    assert torch.equal(handle.doc_scores_window(rows, temperature=0.05), want)
+    other = rows.clone()
+    assert torch.equal(handle.doc_scores_window(other, temperature=0.05), want)          # another tensor object: from the partials
+    assert torch.allclose(handle.doc_scores_window(rows, temperature=0.1), want * 0.5, rtol=1e-6)
+    labels = lay.labels.to(DEV)
+    l1 = br.compute_auxiliary_attention_loss(handle, labels, lay.valid.to(DEV), return_logits=True)
+    hint = br.bracket_rows(labels, R)
+    _, h2 = br.blockrank_attention_forward(Layer(), q, k, v, mask, scale, layers_to_return_scores=[3], score_rows_hint=hint, qk_fp8=qk_fp8)
+    l2 = br.compute_auxiliary_attention_loss(h2, labels, lay.valid.to(DEV), return_logits=True, rows=hint)
+    assert l2 is h2.ranked[2] and torch.equal(l1, l2)
+
+
+def test_score_reduction_in_the_attention_call_argument_errors():
+    lay = synthetic.make_layout([[20, 30, 25, 18]])
+    q, k, v = synthetic.random_qkv(lay, 4, 2, 64, torch.bfloat16, DEV, seed=1)
+    mask = br.BlockMask(lay.valid.to(DEV), torch.bfloat16)
+    rows = torch.zeros((1, 2), dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError):
+        br.blockrank_attention(q, k, v, mask, 0.125, rank_rows=rows)
+    with pytest.raises(AssertionError, match="rows not supported"):
+        br.blockrank_attention(q, k, v, mask, 0.125, score_rows=16, rank_rows=torch.zeros((1, 17), dtype=torch.int32, device=DEV))
