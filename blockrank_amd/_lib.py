@@ -53,7 +53,7 @@ SIGNATURES = {
                                       c_int, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),
     "br_prefill_fwd_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_size_t, c_void_p, c_void_p]),
-    "br_prefill_fp8qk_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int64]),
+    "br_prefill_fp8qk_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int64]),
     "br_prefill_fwd_fp8qk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_void_p, c_size_t,
                                      c_int, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p]),

@@ -364,7 +364,7 @@ def blockrank_attention(
             if query.dtype != torch.bfloat16 or D != 128:
                 raise NotImplementedError("the fp8 Q K^T variant takes bfloat16 inputs with head dim 128")
             opt.fp8_tokens = S if packed else B * S
-            ws_bytes = lib.br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, opt.fp8_tokens)
+            ws_bytes = lib.br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, M, opt.fp8_tokens)
         ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
         if q_rope is not None:
             cos, sin = q_rope

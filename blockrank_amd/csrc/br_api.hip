@@ -194,10 +194,10 @@ size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows) {
 
 static size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int64_t tokens) {
+size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int M, int64_t tokens) {
     const size_t base = br_prefill_workspace_bytes(B, Nq, Nkv, D);
-    if (base == 0 || tokens <= 0) return 0;
-    return up256(base) + up256((size_t)Nkv * tokens * D) + 2 * up256((size_t)B * Nkv * 4);
+    if (base == 0 || tokens <= 0 || M <= 0) return 0;
+    return up256(base) + up256((size_t)Nkv * tokens * D) + up256((size_t)B * M * Nkv * 4) + up256((size_t)B * Nkv * 4);
 }
 
 // Everything optional about a forward call, in one place (the entry points below fill in what they expose).
@@ -277,7 +277,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     make_geom(Nq, Nkv, &g, &nw);
     if (fp8_tokens > 0 && (dtype != BR_DTYPE_BF16 || D != 128))
         return fail(BR_ERR_ARG, "the fp8 Q K^T variant takes bf16 inputs with head dim 128");
-    const size_t need = fp8_tokens > 0 ? br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, fp8_tokens) : br_prefill_workspace_bytes(B, Nq, Nkv, D);
+    const size_t need = fp8_tokens > 0 ? br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, M, fp8_tokens) : br_prefill_workspace_bytes(B, Nq, Nkv, D);
     if (!workspace || workspace_bytes < need) return fail(BR_ERR_SPACE, "workspace holds %zu bytes, %zu needed", workspace_bytes, need);
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
@@ -336,7 +336,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         void* k8 = w;
         w += up256((size_t)Nkv * fp8_tokens * D);
         unsigned* amax = reinterpret_cast<unsigned*>(w);
-        w += up256((size_t)B * Nkv * 4);
+        w += up256((size_t)B * M * Nkv * 4);
         float* scales = reinterpret_cast<float*>(w);
         const long long sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
         br_launch_quantize_fp8(k, plan, k8, amax, scales, sk, k8_b, k8_h, B, Nkv, M, H, D, s);

@@ -180,10 +180,10 @@ int br_prefill_fwd_ex(const void* q, const void* k, const void* v, void* out, co
                       const int64_t* out_strides, float scale, int dtype, void* workspace, size_t workspace_bytes,
                       const BrPrefillOptions* opt, void* stream);
 
-/* Bytes of scratch br_prefill_fwd_fp8qk needs: the split-KV partials plus the quantised K and its scales.
- * tokens: length of the token axis summed over the batch (B*M*H for the padded layout, the number of
- * real tokens for a packed one). */
-size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int64_t tokens);
+/* Bytes of scratch br_prefill_fwd_fp8qk needs: the split-KV partials plus the quantised K, the per-block maxima
+ * (B*M*Nkv) and the scales.  tokens: length of the token axis summed over the batch (B*M*H for the padded layout,
+ * the number of real tokens for a packed one). */
+size_t br_prefill_fp8qk_workspace_bytes(int B, int Nq, int Nkv, int D, int M, int64_t tokens);
 
 /* br_prefill_fwd_scores with the Q K^T products of the prefix and document blocks computed in fp8 e4m3
  * and P V in bf16.  q, k, v, out are bf16 as in br_prefill_fwd.  K is first quantised per (sequence, kv

@@ -43,7 +43,7 @@ def test_pure_host_entry_points():
     assert lib.br_plan_ints(0, 22, 160, 32, 8) == 0
     assert lib.br_prefill_workspace_bytes(4, 32, 8, 128) == 4 * 32 * 8 * 128 * 130 * 4
     assert lib.br_doc_scores_workspace_bytes(4, 32, 22, 2) == 4 * 32 * 2 * 20 * 2 * 4
-    assert lib.br_prefill_fp8qk_workspace_bytes(4, 32, 8, 128, 4 * 3520) > lib.br_prefill_workspace_bytes(4, 32, 8, 128)
+    assert lib.br_prefill_fp8qk_workspace_bytes(4, 32, 8, 128, 22, 4 * 3520) > lib.br_prefill_workspace_bytes(4, 32, 8, 128)
     # backward: fp32 sums of the query block's dQ rows and of the prefix keys' dK / dV, rounded up to 256 bytes, then one
     # float per token slot and query head (delta)
     assert lib.br_prefill_bwd_workspace_bytes(4, 32, 8, 160, 128, 4 * 3520) == 4 * (32 + 16) * 160 * 128 * 4 + 4 * 3520 * 32 * 4
