@@ -599,12 +599,10 @@ def last_block_logits(query, key, block_mask, rows, scaling: float, neg: Optiona
 class _LastLogitsWithGrad(torch.autograd.Function):
     """last_block_logits with a backward: s[b,n,r,k] = scaling * q[b,n,row_r] . k[b,n//G,k] + constant, so
     dq[row_r] = scaling * sum_k ds k and dk[k] = scaling * sum_{n in group, r} ds q[row_r] - two small products
-    over the R score rows, done with torch matmuls (padded layout only)."""
+    over the R score rows (br_last_block_logits_bwd; padded and packed layouts)."""
 
     @staticmethod
     def forward(ctx, query, key, bm, rows, scaling, neg):
-        if bm.packed:
-            raise NotImplementedError("gradients of the score logits need the padded (B, M, H) layout")
         ctx.save_for_backward(query, key, rows)
         ctx.bm, ctx.scaling = bm, float(scaling)
         return last_block_logits(query.detach(), key.detach(), bm, rows, scaling, neg=neg)
@@ -614,17 +612,31 @@ class _LastLogitsWithGrad(torch.autograd.Function):
     def backward(ctx, ds):
         query, key, rows = ctx.saved_tensors
         bm = ctx.bm
-        B, Nq, S, D = query.shape
-        Nkv = key.shape[1]
-        G, R = Nq // Nkv, rows.shape[1]
-        tok = ((bm.M - 1) * bm.H + rows.long())[:, None, :, None].expand(B, Nq, R, D)          # token index of each score row
-        ds5 = ds.float().reshape(B, Nkv, G, R, S)
-        q_rows = query.detach().gather(2, tok).float().reshape(B, Nkv, G, R, D)
-        dq_rows = ctx.scaling * torch.einsum("bkgrs,bksd->bkgrd", ds5, key.detach().float())
-        dk = ctx.scaling * torch.einsum("bkgrs,bkgrd->bksd", ds5, q_rows)
-        dq = torch.zeros((B, Nq, S, D), dtype=torch.float32, device=query.device)
-        dq.scatter_add_(2, tok, dq_rows.reshape(B, Nq, R, D))
-        return dq.to(query.dtype), dk.to(key.dtype), None, None, None, None
+        _, q, k, rows, (B, Nq, Nkv, S, D) = _score_args(query.detach(), key.detach(), bm, rows)
+        R = rows.shape[1]
+        lib = _lib.load()
+        dev = query.device
+        ds = ds.float().contiguous()
+        Bt = q.shape[0]
+        with torch.cuda.device(dev):
+            plan = bm.plan(Nq, Nkv)
+            # gradients in the (B, S, heads, D) layout the projections' outputs have, returned as head-transposed views
+            dq = torch.zeros((Bt, S, Nq, D), dtype=q.dtype, device=dev)
+            dk = None
+            for r0 in range(0, R, 16):                                  # the kernels take up to 16 rows per call
+                rws = rows[:, r0:r0 + 16].contiguous()
+                dsc = ds if R <= 16 else ds[:, :, r0:r0 + 16].contiguous()
+                dki = torch.empty((Bt, S, Nkv, D), dtype=k.dtype, device=dev)
+                dqi = dq if r0 == 0 else torch.zeros_like(dq)
+                _lib.check(lib.br_last_block_logits_bwd(
+                    dsc.data_ptr(), q.data_ptr(), k.data_ptr(), plan.data_ptr(), rws.data_ptr(), rws.shape[1], B, Nq, Nkv, bm.M, bm.H, D,
+                    _lib.strides3(q, bm.packed), _lib.strides3(k, bm.packed), ctx.scaling, _DTYPE_CODE[q.dtype],
+                    dqi.data_ptr(), _lib.strides3(dqi.transpose(1, 2), bm.packed), dki.data_ptr(), _lib.strides3(dki.transpose(1, 2), bm.packed),
+                    _stream_ptr(dev)))
+                if r0 > 0:
+                    dq += dqi
+                dk = dki if dk is None else dk + dki
+        return dq.transpose(1, 2), dk.transpose(1, 2), None, None, None, None
 
 
 def blockrank_attention_forward(

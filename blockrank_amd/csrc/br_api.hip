@@ -30,6 +30,9 @@ int br_launch_last_logits(const void* q, const void* k, const int* plan, const i
                           const long long* sk, int B, int Nq, int Nkv, int M, int H, int D, int R, int T, float scale,
                           float neg, int dtype, hipStream_t stream);
 
+int br_launch_last_logits_bwd(const float* ds, const void* q, const void* k, const int* plan, const int* rows, void* dq, void* dk,
+                              const long long* sq, const long long* sk, const long long* sdq, const long long* sdk, int B, int Nq,
+                              int Nkv, int M, int H, int D, int R, int T, float scale, int dtype, hipStream_t stream);
 int br_launch_bwd(const BrBwdParams& p, int D, int NW, int n_cu, hipStream_t stream);
 int br_launch_rmsnorm(const void* x, const void* w, void* out, long long rows, int hidden, long long sx, long long so, float eps, int dtype,
                       int n_cu, hipStream_t stream);
@@ -590,6 +593,28 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
                           dtype, static_cast<hipStream_t>(stream));
     return check_launch("logits launch");
 }
+
+int br_last_block_logits_bwd(const float* dlogits, const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B,
+                             int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, float scale,
+                             int dtype, void* dq, const int64_t* dq_strides, void* dk, const int64_t* dk_strides, void* stream) {
+    int rc = check_scores(q, k, plan, rows, R, B, Nq, Nkv, M, H, D, q_strides, k_strides, dtype);
+    if (rc) return rc;
+    if (!dlogits || !dq || !dk || !dq_strides || !dk_strides) return fail(BR_ERR_ARG, "null pointer");
+    const long long sq[3] = {q_strides[0], q_strides[1], q_strides[2]};
+    const long long sk[3] = {k_strides[0], k_strides[1], k_strides[2]};
+    const long long sdq[3] = {dq_strides[0], dq_strides[1], dq_strides[2]};
+    const long long sdk[3] = {dk_strides[0], dk_strides[1], dk_strides[2]};
+    for (const long long* st : {sdq, sdk})
+        for (int i = 0; i < 3; ++i)
+            if (st[i] < 0) return fail(BR_ERR_ARG, "negative gradient stride");
+    BrGeom g;
+    int nw;
+    make_geom(Nq, Nkv, &g, &nw);
+    br_launch_last_logits_bwd(dlogits, q, k, plan, rows, dq, dk, sq, sk, sdq, sdk, B, Nq, Nkv, M, H, D, R, br_tokens_per_tile(g), scale,
+                              dtype, static_cast<hipStream_t>(stream));
+    return check_launch("score-logit gradient launch");
+}
+
 
 int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
                int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* cs_strides, int dtype, void* stream) {

@@ -280,6 +280,158 @@ __global__ __launch_bounds__(256) void br_last_logits_kernel(BrScoreParams p) {
     }
 }
 
+
+// ---- gradient of br_last_logits_kernel ----
+// s[b,n,r,key] = scale * q[b,n,row_r] . k[b,n/G,key] + constant for real rows and real keys (the additive mask is a
+// constant, so disallowed real keys carry gradient like the reference's additive-mask logits do); slots without a token
+// and rows that are padding do not depend on q or k at all.
+struct BrLogitsBwdParams {
+    const float* ds;        // (B, Nq, R, M*H) gradient of the logits
+    const void* q;
+    const void* k;
+    const int* plan;
+    const int* rows;        // (B, R) positions inside the query block
+    void* dq;               // caller-zeroed; only the chosen rows are written
+    void* dk;               // every key token is written
+    long long sq_b, sq_h, sq_t, sk_b, sk_h, sk_t;
+    long long dq_b, dq_h, dq_t, dk_b, dk_h, dk_t;
+    int B, Nq, Nkv, M, H, D, R, T;
+    float scale;
+};
+
+template <typename T>
+__device__ inline void store_row_piece(T* dst, const float* x, int n);
+template <>
+__device__ inline void store_row_piece<float>(float* dst, const float* x, int n) {
+    for (int i = 0; i < n; ++i) dst[i] = x[i];
+}
+template <>
+__device__ inline void store_row_piece<__bf16>(__bf16* dst, const float* x, int n) {
+    for (int i = 0; i < n; ++i) dst[i] = (__bf16)x[i];
+}
+
+// dk[key] = scale * sum over the kv head's query heads n and rows r of ds[n, r, key] * q[n, row_r].  One thread per key
+// slot, the whole row of D sums in its registers; the query vectors go through LDS sixteen (head, row) pairs at a time.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void br_last_logits_bwd_dk_kernel(BrLogitsBwdParams p) {
+    __shared__ float qs[kQR * D];
+    __shared__ int ok[kQR];
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.T);
+    const int b = blockIdx.z, kvh = blockIdx.y;
+    const int G = p.Nq / p.Nkv;
+    const int S = p.M * p.H;
+    const int hc = kQR / p.R;                                  // heads per pass
+    const int key = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool in_range = key < S;
+    const int kk = in_range ? key : 0;
+    const int blk = kk / p.H, j = kk - blk * p.H;
+    const int st = pv.start[b * p.M + blk], ln = pv.len[b * p.M + blk];
+    const bool kvalid = in_range && j >= st && j < st + ln;
+    const bool packed = pv.hdr[BR_PH_PACKED] != 0;
+    float acc[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) acc[d] = 0.f;
+    BrScoreParams sp;                                           // what stage_queries reads
+    sp.q = p.q; sp.rows = p.rows; sp.sq_b = p.sq_b; sp.sq_h = p.sq_h; sp.sq_t = p.sq_t; sp.M = p.M; sp.R = p.R; sp.D = D;
+    for (int h0 = 0; h0 < G; h0 += hc) {
+        const int nheads = h0 + hc <= G ? hc : G - h0;
+        __syncthreads();
+        stage_queries<T>(sp, pv, b, kvh * G + h0, nheads, p.scale, qs, ok);
+        __syncthreads();
+        if (kvalid) {
+            for (int jq = 0; jq < nheads * p.R; ++jq) {
+                const int h = jq / p.R, r = jq - h * p.R;
+                const float w = p.ds[(((long long)b * p.Nq + kvh * G + h0 + h) * p.R + r) * S + key];
+                const float* qv = qs + jq * D;
+#pragma unroll
+                for (int d = 0; d < D; ++d) acc[d] = fmaf(w, qv[d], acc[d]);
+            }
+        }
+    }
+    if (!in_range || (packed && !kvalid)) return;              // a packed layout has no storage for empty slots
+    const long long tokn = kvalid ? pv.tok[b * p.M + blk] + j - st : (long long)blk * p.H + j;
+    T* dst = reinterpret_cast<T*>(p.dk) + (long long)b * p.dk_b + (long long)kvh * p.dk_h + tokn * p.dk_t;
+    store_row_piece<T>(dst, acc, D);
+}
+
+// dq[row_r] = scale * sum over the real keys of ds[n, r, key] * k[key].  One workgroup per (sequence, head): thread =
+// (key phase, dim), sixteen row sums in registers; the ds values and the slot -> token map of 256 keys at a time in LDS.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void br_last_logits_bwd_dq_kernel(BrLogitsBwdParams p) {
+    constexpr int NPH = 256 / D;                               // key phases
+    constexpr int CH = 256;                                    // keys per chunk
+    __shared__ float dsl[kQR * CH];
+    __shared__ int tokl[CH];
+    static_assert(NPH * kQR * D <= kQR * CH, "the phase reduction reuses the ds buffer");
+    const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.T);
+    const int b = blockIdx.y, n = blockIdx.x;
+    const int G = p.Nq / p.Nkv, kvh = n / G;
+    const int S = p.M * p.H;
+    const int d = threadIdx.x % D, ph = threadIdx.x / D;
+    const T* kb = reinterpret_cast<const T*>(p.k) + (long long)b * p.sk_b + (long long)kvh * p.sk_h + d;
+    float acc[kQR];
+#pragma unroll
+    for (int r = 0; r < kQR; ++r) acc[r] = 0.f;
+    for (int s0 = 0; s0 < S; s0 += CH) {
+        __syncthreads();
+        {
+            const int key = s0 + threadIdx.x;
+            int tk = -1;
+            if (key < S) {
+                const int blk = key / p.H, j = key - blk * p.H;
+                const int st = pv.start[b * p.M + blk], ln = pv.len[b * p.M + blk];
+                if (j >= st && j < st + ln) tk = pv.tok[b * p.M + blk] + j - st;
+            }
+            tokl[threadIdx.x] = tk;
+            for (int r = 0; r < p.R; ++r)
+                dsl[r * CH + threadIdx.x] = key < S ? p.ds[(((long long)b * p.Nq + n) * p.R + r) * S + key] : 0.f;
+        }
+        __syncthreads();
+        constexpr int U = 8;
+        for (int i0 = ph; i0 < CH; i0 += NPH * U) {
+            float kv[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = i0 + u * NPH;
+                const int tk = i < CH ? tokl[i] : -1;
+                kv[u] = tk >= 0 ? (float)kb[(long long)tk * p.sk_t] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = i0 + u * NPH;
+                if (i < CH) {
+#pragma unroll
+                    for (int r = 0; r < kQR; ++r)
+                        if (r < p.R) acc[r] = fmaf(dsl[r * CH + i], kv[u], acc[r]);
+                }
+            }
+        }
+    }
+    // add the key phases up (in dsl, free now), then one thread per (row, dim) writes the row - rows named twice are
+    // summed into their first occurrence
+    __syncthreads();
+    float* red2 = dsl;                                          // [NPH][R][D] <= 16 * 256 floats
+    for (int r = 0; r < p.R; ++r) red2[(ph * kQR + r) * D + d] = acc[r];
+    __syncthreads();
+    const int m = p.M - 1;
+    const int st = pv.start[b * p.M + m], ln = pv.len[b * p.M + m], tk0 = pv.tok[b * p.M + m];
+    for (int idx = threadIdx.x; idx < p.R * D; idx += blockDim.x) {
+        const int r = idx / D, dd = idx - r * D;
+        const int pos = p.rows[b * p.R + r];
+        if (pos < st || pos >= st + ln) continue;              // a padded row: its logits do not depend on q
+        bool first = true;
+        for (int r2 = 0; r2 < r; ++r2) first = first && p.rows[b * p.R + r2] != pos;
+        if (!first) continue;
+        float v = 0.f;
+        for (int r2 = r; r2 < p.R; ++r2)
+            if (p.rows[b * p.R + r2] == pos)
+                for (int q = 0; q < NPH; ++q) v += red2[(q * kQR + r2) * D + dd];
+        T* dst = reinterpret_cast<T*>(p.dq) + (long long)b * p.dq_b + (long long)n * p.dq_h + (long long)(tk0 + pos - st) * p.dq_t + dd;
+        const float out = v * p.scale;
+        store_row_piece<T>(dst, &out, 1);
+    }
+}
+
 }  // namespace
 
 // dtype: 0 fp32, 1 bf16
@@ -358,3 +510,30 @@ int br_launch_doc_scores_tiles(const float* part, const int* plan, const int* ro
     return 0;
 }
 
+int br_launch_last_logits_bwd(const float* ds, const void* q, const void* k, const int* plan, const int* rows, void* dq, void* dk,
+                              const long long* sq, const long long* sk, const long long* sdq, const long long* sdk, int B, int Nq,
+                              int Nkv, int M, int H, int D, int R, int T, float scale, int dtype, hipStream_t stream) {
+    BrLogitsBwdParams p;
+    p.ds = ds; p.q = q; p.k = k; p.plan = plan; p.rows = rows; p.dq = dq; p.dk = dk;
+    p.sq_b = sq[0]; p.sq_h = sq[1]; p.sq_t = sq[2];
+    p.sk_b = sk[0]; p.sk_h = sk[1]; p.sk_t = sk[2];
+    p.dq_b = sdq[0]; p.dq_h = sdq[1]; p.dq_t = sdq[2];
+    p.dk_b = sdk[0]; p.dk_h = sdk[1]; p.dk_t = sdk[2];
+    p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H; p.D = D; p.R = R; p.T = T; p.scale = scale;
+    const int S = M * H;
+    dim3 gk((S + 255) / 256, Nkv, B), gq(Nq, B);
+    if (dtype == 0 && D == 64) {
+        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<float, 64>), gk, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<float, 64>), gq, dim3(256), 0, stream, p);
+    } else if (dtype == 0) {
+        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<float, 128>), gk, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<float, 128>), gq, dim3(256), 0, stream, p);
+    } else if (D == 64) {
+        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<__bf16, 64>), gk, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<__bf16, 64>), gq, dim3(256), 0, stream, p);
+    } else {
+        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<__bf16, 128>), gk, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<__bf16, 128>), gq, dim3(256), 0, stream, p);
+    }
+    return 0;
+}

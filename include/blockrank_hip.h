@@ -241,6 +241,19 @@ int br_last_block_logits(const void* q, const void* k, const int32_t* plan, cons
                          int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
                          float scale, float neg, int dtype, float* logits, void* stream);
 
+/* Gradient of br_last_block_logits with respect to q and k, given the gradient of its output: what torch autograd
+ * derives for the s_last tensor of the reference's trainable hooks (blockrank_std_attention.py:242-262, :639-645), through
+ * which the auxiliary attention loss trains (trainer.py:91-101, losses.py:53-74).
+ *   dlogits (B, Nq, R, M*H) fp32.  Real rows against real keys carry gradient (also keys the row may not see: the mask is
+ *   an added constant); slots without a token and rows that are padding carry none, as in br_last_block_logits.
+ *   dq: a zero-filled tensor addressed like q (element strides dq_strides); only the R chosen rows of every head are
+ *   written (rows named twice are summed).  dk: addressed like k (dk_strides); every key token is written (in the padded
+ *   layout the empty slots get zero), so it needs no initialisation.  dtype of q, k, dq, dk: 0 fp32, 1 bf16.
+ *   Padded and packed layouts; R <= 16 per call. */
+int br_last_block_logits_bwd(const float* dlogits, const void* q, const void* k, const int32_t* plan, const int32_t* rows, int R, int B,
+                             int Nq, int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, float scale,
+                             int dtype, void* dq, const int64_t* dq_strides, void* dk, const int64_t* dk_strides, void* stream);
+
 /* Rotary position embedding of Q and K in one pass, the step in front of every attention call:
  * out = x * cos + rotate_half(x) * sin, rotate_half(x) = (-x[D/2:], x[:D/2]).  Replaces apply_rotary_pos_emb of
  * the Hugging Face model the reference ranks with (transformers models/mistral/modeling_mistral.py,

@@ -232,3 +232,88 @@ def test_score_reduction_in_the_attention_call_argument_errors():
         br.blockrank_attention(q, k, v, mask, 0.125, rank_rows=rows)
     with pytest.raises(AssertionError, match="rows not supported"):
         br.blockrank_attention(q, k, v, mask, 0.125, score_rows=16, rank_rows=torch.zeros((1, 17), dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("dtype,Nq,Nkv,D,tol", [(torch.float32, 8, 2, 64, 2e-5), (torch.bfloat16, 8, 2, 128, 1.2e-2), (torch.float32, 6, 6, 128, 2e-5)])
+def test_gradient_of_the_last_block_logits(dtype, Nq, Nkv, D, tol):
+    """LastBlockScores.dense() with gradients: dq and dk from the HIP kernels against torch autograd of the closed form
+    s = scale * q_row . k over real rows and real keys (fp32: to rounding; bf16: to the rounding of the stored result),
+    padded and packed layouts, 16 default rows; a loss through compute_auxiliary_attention_loss on top."""
+    lay = synthetic.make_layout([[9, 30, 0, 17, 20], [12, 5, 33, 8, 13]])
+    R, scale = 16, 0.17
+    q0, k0, _ = synthetic.random_qkv(lay, Nq, Nkv, D, dtype, DEV, seed=5)
+    valid = lay.valid.to(DEV)
+    B, S, H, M = lay.B, lay.S, lay.H, lay.lengths.shape[1]
+    G = Nq // Nkv
+    g = torch.Generator().manual_seed(2)
+    ds = torch.randn(B, Nq, R, S, generator=g).to(DEV)
+
+    # closed form in float64 on the padded layout
+    qr = q0.double().clone().requires_grad_(True)
+    kr = k0.double().clone().requires_grad_(True)
+    vrow = valid.reshape(B, S)
+    rows_tok = torch.arange(S - R, S, device=DEV)
+    row_real = vrow[:, rows_tok]                                            # (B, R)
+    s_ref = scale * torch.einsum("bnrd,bnsd->bnrs", qr[:, :, rows_tok], kr.repeat_interleave(G, dim=1))
+    s_ref = s_ref * (row_real[:, None, :, None] & vrow[:, None, None, :])   # padded rows / empty slots: constants
+    (s_ref * ds.double()).sum().backward()
+
+    def run(bm, q, k):
+        q = q.clone().requires_grad_(True)
+        k = k.clone().requires_grad_(True)
+        h = br.LastBlockScores(q, k, bm, scale, R)
+        assert h.needs_grad()
+        out = h.dense()
+        assert out.shape == (B, Nq, R, S) and out.requires_grad
+        (out * ds).sum().backward()
+        return q.grad, k.grad
+
+    dq, dk = run(br.BlockMask(valid, dtype), q0, k0)
+    real = vrow[:, None, :, None]
+    for got, want, name in ((dq, qr.grad, "dq"), (dk, kr.grad, "dk")):
+        want = want * real                                                   # (the closed form has zeros there already)
+        err = (got.double() - want).abs().max().item() / max(want.abs().max().item(), 1e-9)
+        assert err <= tol, f"{name}: {err}"
+        assert (got * ~real).abs().max().item() == 0.0, f"{name}: padded slots must be zero"
+
+    # packed layout: the same numbers on the real tokens
+    from tests.test_gpu_packed import _pack
+    lengths = torch.as_tensor(lay.lengths, dtype=torch.int32, device=DEV)
+    packed = br.BlockMask.from_lengths(lengths, H=H, packed=True, dtype=dtype)
+    dqp, dkp = run(packed, _pack(q0, lay.valid), _pack(k0, lay.valid))
+    assert torch.equal(dqp, _pack(dq, lay.valid)) and torch.equal(dkp, _pack(dk, lay.valid))
+
+    # through the loss API (the training path of trainer.py:91-101)
+    q = q0.clone().requires_grad_(True)
+    k = k0.clone().requires_grad_(True)
+    h = br.LastBlockScores(q, k, br.BlockMask(valid, dtype), scale, R)
+    loss, acc = br.compute_auxiliary_attention_loss(h, lay.labels.to(DEV), valid, answer_ids=torch.tensor([[1], [0]], device=DEV))
+    loss.backward()
+    assert torch.isfinite(q.grad).all() and torch.isfinite(k.grad).all() and q.grad.abs().max() > 0 and k.grad.abs().max() > 0
+
+
+def test_gradient_of_the_logits_rows_named_twice():
+    """The C entry with a row given twice: its two gradient rows add up in dq (one row of the tensor)."""
+    from blockrank_amd import _lib
+    from blockrank_amd.attention import _stream_ptr
+    lay = synthetic.make_layout([[8, 20, 12, 16]])
+    Nq, Nkv, D, scale = 4, 2, 64, 0.2
+    q, k, _ = synthetic.random_qkv(lay, Nq, Nkv, D, torch.float32, DEV, seed=1)
+    bm = br.BlockMask(lay.valid.to(DEV), torch.float32)
+    rows = torch.tensor([[lay.H - 3, lay.H - 1, lay.H - 3]], dtype=torch.int32, device=DEV)   # real positions of the query block
+    ds = torch.randn(1, Nq, 3, lay.S, generator=torch.Generator().manual_seed(3)).to(DEV)
+    lib = _lib.load()
+    plan = bm.plan(Nq, Nkv)
+    dq = torch.zeros(1, lay.S, Nq, D, device=DEV)
+    dk = torch.empty(1, lay.S, Nkv, D, device=DEV)
+    _lib.check(lib.br_last_block_logits_bwd(ds.data_ptr(), q.data_ptr(), k.data_ptr(), plan.data_ptr(), rows.data_ptr(), 3, 1, Nq, Nkv, bm.M, bm.H, D,
+                                            _lib.strides3(q), _lib.strides3(k), scale, 0, dq.data_ptr(), _lib.strides3(dq.transpose(1, 2)),
+                                            dk.data_ptr(), _lib.strides3(dk.transpose(1, 2)), _stream_ptr(torch.device(DEV))))
+    vrow = lay.valid.reshape(1, lay.S).to(DEV)
+    kk = (k * vrow[:, None, :, None]).repeat_interleave(Nq // Nkv, dim=1)
+    per_row = scale * torch.einsum("bnrs,bnsd->bnrd", ds, kk)                 # (1, Nq, 3, D)
+    tok = 3 * lay.H + rows[0].long()
+    want = torch.zeros_like(dq)
+    want[0, tok[0]] = per_row[0, :, 0] + per_row[0, :, 2]
+    want[0, tok[1]] = per_row[0, :, 1]
+    torch.testing.assert_close(dq, want, rtol=1e-5, atol=1e-5)
