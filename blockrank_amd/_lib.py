@@ -13,6 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libblockrank_hip.so"
 
 BR_DTYPE_F32 = 0
 BR_DTYPE_BF16 = 1
+BR_DTYPE_F16 = 2
 
 BR_ERR_ARG = 1
 BR_ERR_SPACE = 2

@@ -33,7 +33,8 @@ STD_IMPL_NAMES = (
 # blockrank_triton_kernel_attention.py:960-965
 TRITON_IMPL_NAMES = ("triton_blockrank", "triton_blockrank_compiled")
 
-_DTYPE_CODE = {torch.float32: _lib.BR_DTYPE_F32, torch.bfloat16: _lib.BR_DTYPE_BF16}
+_DTYPE_CODE = {torch.float32: _lib.BR_DTYPE_F32, torch.bfloat16: _lib.BR_DTYPE_BF16, torch.float16: _lib.BR_DTYPE_F16}
+_HALF = (torch.bfloat16, torch.float16)      # the MFMA kernels' input types
 
 
 def _env_flag(name: str) -> bool:
@@ -335,10 +336,10 @@ def blockrank_attention(
         assert Bt == B, "attention mask batch size does not match query"
     assert key.shape == (Bt, Nkv, S, D) and value.shape == (Bt, Nkv, S, D), "key/value must be (B, Nkv, S, D)"
     if query.dtype not in _DTYPE_CODE:
-        raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
+        raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16, float16 and float32 are)")
     assert key.dtype == query.dtype and value.dtype == query.dtype, "query, key and value must share a dtype"
-    if q_rope is not None and (query.dtype != torch.bfloat16 or qk_fp8):
-        raise NotImplementedError("the rotary embedding inside the attention kernel takes bfloat16 inputs and not the fp8 variant")
+    if q_rope is not None and (query.dtype not in _HALF or qk_fp8):
+        raise NotImplementedError("the rotary embedding inside the attention kernel takes 16-bit inputs and not the fp8 variant")
     if torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad):
         if query.dtype != torch.bfloat16 or qk_fp8 or score_rows > 0 or q_rope is not None:
             # same contract as the reference's kernelised path (blockrank_triton_kernel_attention.py:759-761)
@@ -401,7 +402,7 @@ def blockrank_attention(
 
 def fused_scores_supported(query: torch.Tensor, block_mask) -> bool:
     """Whether blockrank_attention(..., score_rows=R) can produce score partials for these inputs."""
-    return query.dtype == torch.bfloat16 and block_mask.M >= 3
+    return query.dtype in _HALF and block_mask.M >= 3
 
 
 def doc_scores_from_partials(partials: torch.Tensor, block_mask, rows: torch.Tensor, score_rows: int, num_heads: int,
@@ -518,7 +519,7 @@ def _score_args(query, key, block_mask, rows, query_block_only=False):
         assert Sq == (bm.H if query_block_only else S), "query must cover the query block only" if query_block_only else \
             "query and key must cover the same tokens"
     if query.dtype not in _DTYPE_CODE:
-        raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16 and float32 are)")
+        raise NotImplementedError(f"dtype {query.dtype} not supported by the HIP kernels (bfloat16, float16 and float32 are)")
     assert rows.dim() == 2 and rows.shape[0] == B, "rows must be (B, R)"
     per16 = 16 // query.element_size()
     q = _dense_last_dim(query, per16)
@@ -704,7 +705,7 @@ def blockrank_attention_forward(
     deferred = getattr(query, "_blockrank_rope", None)
     q_rope = None
     if deferred is not None:
-        if want or qk_fp8 or needs_grad or query.dtype != torch.bfloat16:
+        if want or qk_fp8 or needs_grad or query.dtype not in _HALF:
             from .rope import rotate_q
             query = rotate_q(query, deferred.cos, deferred.sin)
         else:

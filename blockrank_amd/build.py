@@ -18,7 +18,7 @@ CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libblockrank_hip.so"
 OBJ_DIR = PKG_DIR / "csrc" / "build"
 
-SOURCES = ["br_api.hip", "br_plan.hip", "br_prefill_mfma.hip", "br_prefill_fp8.hip", "br_rope.hip", "br_bwd.hip", "br_norm_act.hip", "br_prefill_f32.hip", "br_scores.hip"]
+SOURCES = ["br_api.hip", "br_plan.hip", "br_prefill_mfma.hip", "br_prefill_f16.hip", "br_prefill_fp8.hip", "br_rope.hip", "br_bwd.hip", "br_norm_act.hip", "br_prefill_f32.hip", "br_scores.hip"]
 
 # -packed-fp32-ops is switched off: the compiler must not form packed fp32 instructions on this target.
 HIPCC_FLAGS = [

@@ -13,6 +13,8 @@ void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int 
                     hipStream_t stream);
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                            hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
+int br_launch_prefill_f16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
+                          hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
 int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                            hipEvent_t ev_start, hipEvent_t ev_stop);
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
@@ -109,7 +111,7 @@ int check_common(int B, int Nq, int Nkv, int M, int H, int D, int dtype) {
     if (B <= 0 || M <= 0 || H <= 0) return fail(BR_ERR_ARG, "B, M and H must be positive (got %d, %d, %d)", B, M, H);
     if (Nq <= 0 || Nkv <= 0 || Nq % Nkv) return fail(BR_ERR_ARG, "Nq=%d must be a positive multiple of Nkv=%d", Nq, Nkv);
     if (D != 64 && D != 128) return fail(BR_ERR_ARG, "head dim %d not supported (64 or 128)", D);
-    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "dtype %d not supported", dtype);
+    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16 && dtype != BR_DTYPE_F16) return fail(BR_ERR_ARG, "dtype %d not supported", dtype);
     return BR_OK;
 }
 
@@ -247,7 +249,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
     if (rc) return rc;
     if (rope_cos || rope_sin) {
-        if (dtype != BR_DTYPE_BF16 || fp8_tokens > 0) return fail(BR_ERR_ARG, "the rotary embedding of Q inside the attention kernel needs the bf16 kernel");
+        if (dtype == BR_DTYPE_F32 || fp8_tokens > 0) return fail(BR_ERR_ARG, "the rotary embedding of Q inside the attention kernel needs the bf16 or fp16 kernel");
         if (!rope_cos || !rope_sin || !rope_strides) return fail(BR_ERR_ARG, "cos, sin and their strides must be given together");
         if (!aligned16(rope_cos) || !aligned16(rope_sin)) return fail(BR_ERR_ARG, "cos and sin must be 16-byte aligned");
         if (rope_strides[0] < 0 || rope_strides[1] < D || rope_strides[0] % 8 || rope_strides[1] % 8 || rope_strides[0] >= (int64_t(1) << 31) ||
@@ -256,7 +258,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     }
     if (lse && (dtype != BR_DTYPE_BF16 || fp8_tokens > 0 || !lse_strides)) return fail(BR_ERR_ARG, "the log-sum-exp output comes from the bf16 kernel only");
     if (score_part) {
-        if (dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "score partials come from the bf16 kernel only; use br_doc_scores");
+        if (dtype == BR_DTYPE_F32) return fail(BR_ERR_ARG, "score partials come from the bf16 / fp16 kernel only; use br_doc_scores");
         if (M < 3) return fail(BR_ERR_ARG, "score partials need at least one document block (M=%d)", M);
         if (score_rows <= 0 || score_rows > H) return fail(BR_ERR_ARG, "score_rows=%d outside 1..H=%d", score_rows, H);
         if (!aligned16(score_part)) return fail(BR_ERR_ARG, "score_part must be 16-byte aligned");
@@ -348,8 +350,9 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         p.qk_scales = scales;
         lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp);
     } else {
-        lrc = dtype == BR_DTYPE_BF16 ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
-                                     : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s, e0, e1);
+        lrc = dtype == BR_DTYPE_BF16  ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
+              : dtype == BR_DTYPE_F16 ? br_launch_prefill_f16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
+                                      : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s, e0, e1);
     }
     if (lrc) return fail(BR_ERR_ARG, "no kernel for head dim %d with %d query heads per kv head", D, g.G);
     return check_launch("prefill launch");
@@ -618,7 +621,7 @@ int br_last_block_logits_bwd(const float* dlogits, const void* q, const void* k,
 
 int br_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
                int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* cs_strides, int dtype, void* stream) {
-    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16) return fail(BR_ERR_ARG, "dtype must be fp32 (0) or bf16 (1)");
+    if (dtype != BR_DTYPE_F32 && dtype != BR_DTYPE_BF16 && dtype != BR_DTYPE_F16) return fail(BR_ERR_ARG, "dtype must be fp32 (0), bf16 (1) or fp16 (2)");
     if (B <= 0 || Nq < 0 || Nkv <= 0 || S <= 0) return fail(BR_ERR_ARG, "B, Nkv and S must be positive, Nq not negative");
     if (D != 64 && D != 128) return fail(BR_ERR_ARG, "head dim %d not supported (64 or 128)", D);
     const int64_t zero3[3] = {0, 0, 0};

@@ -35,9 +35,23 @@
 
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// The 16-bit element type of Q, K, V and the output is a property of the translation unit: BR_E16 is __bf16 unless the
+// including file defines it as _Float16 (with BR_E16_IS_F16).  Same layouts, same kernels; the matrix and dot-product
+// instructions are the ones of that type.
+#ifndef BR_E16
+#define BR_E16 __bf16
+#endif
+typedef float br_f32x16 __attribute__((ext_vector_type(16)));
+typedef BR_E16 e16x8 __attribute__((ext_vector_type(8)));
+typedef BR_E16 e16x4 __attribute__((ext_vector_type(4)));
+typedef BR_E16 e16x2 __attribute__((ext_vector_type(2)));
+#ifdef BR_E16_IS_F16
+__device__ inline br_f32x16 br_mma16(e16x8 a, e16x8 b, br_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+__device__ inline float br_dot2(e16x2 a, e16x2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
+#else
+__device__ inline br_f32x16 br_mma16(e16x8 a, e16x8 b, br_f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+__device__ inline float br_dot2(e16x2 a, e16x2 b, float c) { return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false); }
+#endif
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -67,8 +81,8 @@ struct Smem {
 };
 
 __device__ inline uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
-__device__ inline bf16x8 as_bf16x8(uint4 u) {
-    union { uint4 u; bf16x8 v; } c;
+__device__ inline e16x8 as_e16x8(uint4 u) {
+    union { uint4 u; e16x8 v; } c;
     c.u = u;
     return c.v;
 }
@@ -272,7 +286,7 @@ __device__ inline void br_pow2_scale(float amax, float& scale, float& inv) {
 
 typedef long k8x8;   // eight fp8 values: one MFMA operand of v_mfma_f32_32x32x16_fp8_fp8
 
-template <bool F8> struct QKFrag { typedef bf16x8 type; };
+template <bool F8> struct QKFrag { typedef e16x8 type; };
 template <> struct QKFrag<true> { typedef k8x8 type; };
 
 template <int D, int NW, bool F8>
@@ -405,22 +419,22 @@ struct Prefill {
         if constexpr (F8) {
             return *reinterpret_cast<const k8x8*>(stage + kb * 32 * SM::rowKB + (L.krd ^ (c << 4)));
         } else {
-            return as_bf16x8(ld16(stage + kb * 32 * SM::rowKB + (L.krd ^ (c << 5))));
+            return as_e16x8(ld16(stage + kb * 32 * SM::rowKB + (L.krd ^ (c << 5))));
         }
     }
     static __device__ inline f32x16 mma_qk(Frag a, Frag b, f32x16 c) {
         if constexpr (F8) {
             return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
         } else {
-            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+            return br_mma16(a, b, c);
         }
     }
     // V^T operand for dims 32d + (lane & 31), keys 16*c2 + 8*lh + 0..7: two transposing reads
-    static __device__ inline bf16x8 read_vt(const char* stage, const Lane& L, int d, int c2) {
+    static __device__ inline e16x8 read_vt(const char* stage, const Lane& L, int d, int c2) {
         const char* vp = stage + L.vrd[d] + c2 * 16 * SM::rowB;
         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)vp);
         s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(__attribute__((address_space(3))) const char*)(vp + 4 * SM::rowB));
-        union { s16x8 s8; bf16x8 b8; } a;
+        union { s16x8 s8; e16x8 b8; } a;
         a.s8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         return a.b8;
     }
@@ -461,7 +475,7 @@ struct Prefill {
             BR_SCHED_FENCE();
         }
         // first V^T operands: their LDS latency passes under the softmax arithmetic
-        bf16x8 va[ND];
+        e16x8 va[ND];
 #pragma unroll
         for (int d = 0; d < ND; ++d) va[d] = read_vt(stage, L, d, 0);
         if (MASK) {
@@ -500,8 +514,8 @@ struct Prefill {
         // denominator then carry the same rounding, and a row whose mass sits on one key reproduces that key's
         // V row exactly instead of V * (rounded p / p).
         float psum = 0.f, psum_t = 0.f;
-        const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
-        bf16x8 pf[2 * NKB];
+        const e16x2 ones2 = {(BR_E16)1.0f, (BR_E16)1.0f};
+        e16x8 pf[2 * NKB];
 #pragma unroll
         for (int c2 = 0; c2 < 2 * NKB; ++c2) {
             f32x8 t;
@@ -510,11 +524,11 @@ struct Prefill {
                 t[e] = __builtin_amdgcn_exp2f(s[c2 >> 1][8 * (c2 & 1) + e] * scale_log2 - m_sub);
                 if (EXACT) psum += t[e];
             }
-            pf[c2] = __builtin_convertvector(t, bf16x8);
-            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 0, 1), ones2, psum_t, false);
-            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 2, 3), ones2, psum_t, false);
-            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 4, 5), ones2, psum_t, false);
-            psum_t = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(pf[c2], pf[c2], 6, 7), ones2, psum_t, false);
+            pf[c2] = __builtin_convertvector(t, e16x8);
+            psum_t = br_dot2(__builtin_shufflevector(pf[c2], pf[c2], 0, 1), ones2, psum_t);
+            psum_t = br_dot2(__builtin_shufflevector(pf[c2], pf[c2], 2, 3), ones2, psum_t);
+            psum_t = br_dot2(__builtin_shufflevector(pf[c2], pf[c2], 4, 5), ones2, psum_t);
+            psum_t = br_dot2(__builtin_shufflevector(pf[c2], pf[c2], 6, 7), ones2, psum_t);
         }
         l_run += psum;
         lt_run += psum_t;
@@ -523,7 +537,7 @@ struct Prefill {
         for (int c2 = 0; c2 < 2 * NKB; ++c2) {
 #pragma unroll
             for (int d = 0; d < ND; ++d) {
-                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d], pf[c2], o[d], 0, 0, 0);
+                o[d] = br_mma16(va[d], pf[c2], o[d]);
                 if (c2 + 1 < 2 * NKB) va[d] = read_vt(stage, L, d, c2 + 1);
             }
         }
@@ -589,7 +603,7 @@ struct Prefill {
         u32x4 qraw[F8 ? D / 16 : 1];       // fp8: the bf16 rows as loaded, converted once they have arrived
         // rotary embedding applied here: the row's cos / sin values for the lane's dims (both halves of the tables)
         constexpr int NRC = F8 ? 1 : D / 32;
-        bf16x8 rcos[2][NRC], rsin[2][NRC];
+        e16x8 rcos[2][NRC], rsin[2][NRC];
         const bool rope = !F8 && p.rope_cos != nullptr && rb_active;
         {
             const char* qrow = reinterpret_cast<const char*>(p.q) +
@@ -603,13 +617,13 @@ struct Prefill {
 #pragma unroll
                 for (int c = 0; c < D / 16; ++c) {
                     if constexpr (F8) qraw[c] = *reinterpret_cast<const u32x4*>(qrow + qoff + c * 32);
-                    else qf[c] = as_bf16x8(ld16(qrow + qoff + c * 32));
+                    else qf[c] = as_e16x8(ld16(qrow + qoff + c * 32));
                 }
             } else {
 #pragma unroll
                 for (int c = 0; c < D / 16; ++c) {
                     if constexpr (F8) qraw[c] = u32x4{0u, 0u, 0u, 0u};
-                    else qf[c] = as_bf16x8(uint4{0u, 0u, 0u, 0u});
+                    else qf[c] = as_e16x8(uint4{0u, 0u, 0u, 0u});
                 }
             }
             if constexpr (!F8) {
@@ -619,10 +633,10 @@ struct Prefill {
                     const char* srow = reinterpret_cast<const char*>(p.rope_sin) + tbl;
 #pragma unroll
                     for (int c = 0; c < NRC; ++c) {
-                        rcos[0][c] = as_bf16x8(ld16(crow + c * 32));
-                        rcos[1][c] = as_bf16x8(ld16(crow + (c + NRC) * 32));
-                        rsin[0][c] = as_bf16x8(ld16(srow + c * 32));
-                        rsin[1][c] = as_bf16x8(ld16(srow + (c + NRC) * 32));
+                        rcos[0][c] = as_e16x8(ld16(crow + c * 32));
+                        rcos[1][c] = as_e16x8(ld16(crow + (c + NRC) * 32));
+                        rsin[0][c] = as_e16x8(ld16(srow + c * 32));
+                        rsin[1][c] = as_e16x8(ld16(srow + (c + NRC) * 32));
                     }
                 }
             }
@@ -694,14 +708,14 @@ struct Prefill {
             if (rope) {
 #pragma unroll
                 for (int c = 0; c < NRC; ++c) {
-                    bf16x8 lo = qf[c], hi = qf[c + NRC];
+                    e16x8 lo = qf[c], hi = qf[c + NRC];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
                         const float x1 = (float)lo[j], x2 = (float)hi[j];
                         const float o1 = x1 * (float)rcos[0][c][j] - x2 * (float)rsin[0][c][j];
                         const float o2 = x2 * (float)rcos[1][c][j] + x1 * (float)rsin[1][c][j];
-                        lo[j] = (__bf16)o1;
-                        hi[j] = (__bf16)o2;
+                        lo[j] = (BR_E16)o1;
+                        hi[j] = (BR_E16)o2;
                     }
                     qf[c] = lo;
                     qf[c + NRC] = hi;
@@ -807,7 +821,7 @@ struct Prefill {
         } else {
             // the last loop iteration ended with a barrier, so the K/V buffers are free: transpose
             // through LDS so that every output row is written as full 16-byte pieces
-            __bf16* Es = reinterpret_cast<__bf16*>(smem + wave * SM::eBytesPerWave);
+            BR_E16* Es = reinterpret_cast<BR_E16*>(smem + wave * SM::eBytesPerWave);
             const float inv = lt_tot > 0.f ? __builtin_amdgcn_rcpf(lt_tot) : 0.f;
             if (p.lse != nullptr && lane_e < 32 && row0 + lane_e < len_m)
                 p.lse[(long long)b * p.lse_b + (long long)head * p.lse_h + qtok0 + row0 + lane_e] = m_run + __builtin_amdgcn_logf(l_tot);
@@ -818,8 +832,8 @@ struct Prefill {
                     for (int q4 = 0; q4 < 4; ++q4) {
                         f32x4 t = {o[d][4 * q4] * inv, o[d][4 * q4 + 1] * inv, o[d][4 * q4 + 2] * inv,
                                    o[d][4 * q4 + 3] * inv};
-                        bf16x4 h4 = __builtin_convertvector(t, bf16x4);
-                        *reinterpret_cast<bf16x4*>(Es + ln * SM::eRow + d * 32 + 8 * q4 + 4 * lh) = h4;
+                        e16x4 h4 = __builtin_convertvector(t, e16x4);
+                        *reinterpret_cast<e16x4*>(Es + ln * SM::eRow + d * 32 + 8 * q4 + 4 * lh) = h4;
                     }
                 // same wave wrote and reads: LDS operations of one wave complete in order; the fence
                 // keeps the compiler from moving the reads above the writes
@@ -991,10 +1005,10 @@ __global__ __launch_bounds__(THREADS) void br_finish_kernel(BrPrefillParams p, i
         const float inv = l > 0.f ? 1.f / l : 0.f;
         if (p.lse != nullptr && cc == 0)
             p.lse[(long long)c.b * p.lse_b + (long long)head * p.lse_h + qtok0 + row] = mmax + __builtin_amdgcn_logf(l);
-        __bf16* dst = reinterpret_cast<__bf16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
+        BR_E16* dst = reinterpret_cast<BR_E16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
                       (long long)(qtok0 + row) * p.so_t;
-        bf16x4 h4 = __builtin_convertvector(acc * inv, bf16x4);
-        *reinterpret_cast<bf16x4*>(dst + cc * 4) = h4;
+        e16x4 h4 = __builtin_convertvector(acc * inv, e16x4);
+        *reinterpret_cast<e16x4*>(dst + cc * 4) = h4;
     }
     // Padded token slots: no kernel computes them, so give them a defined value (zero).  The prefill kernel
     // does that for the documents it has items for; what is left here are the prefix, the query block and
@@ -1011,7 +1025,7 @@ __global__ __launch_bounds__(THREADS) void br_finish_kernel(BrPrefillParams p, i
         if (ln != 0 && mm > 0 && mm < p.M - 1) continue;
         const int npad = p.H - ln;
         constexpr int CP8 = D / 8;
-        __bf16* obase = reinterpret_cast<__bf16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
+        BR_E16* obase = reinterpret_cast<BR_E16*>(p.out) + (long long)b * p.so_b + (long long)head * p.so_h;
         for (int idx = lane; idx < npad * CP8; idx += 64) {
             int r = idx / CP8, c8 = idx - r * CP8;
             int pos = r < st ? r : r + ln;

@@ -24,6 +24,7 @@ struct BrRopeParams {
 
 template <typename T> struct Vec16;
 template <> struct Vec16<__bf16> { static constexpr int N = 8; };
+template <> struct Vec16<_Float16> { static constexpr int N = 8; };
 template <> struct Vec16<float> { static constexpr int N = 4; };
 
 template <typename T>
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) void br_rope_kernel(BrRopeParams p) {
 
 }  // namespace
 
-// dtype: 0 fp32, 1 bf16 (q, k, cos, sin and the outputs alike).
+// dtype: 0 fp32, 1 bf16, 2 fp16 (q, k, cos, sin and the outputs alike).
 int br_launch_rope(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Nq, int Nkv, int S,
                    int D, const long long* sq, const long long* sk, const long long* sc, int dtype, int n_cu, hipStream_t stream) {
     BrRopeParams p;
@@ -101,7 +102,9 @@ int br_launch_rope(const void* q, const void* k, const void* cos, const void* si
     if (blocks < 1) blocks = 1;
     if (dtype == 0)
         hipLaunchKernelGGL(br_rope_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
-    else
+    else if (dtype == 1)
         hipLaunchKernelGGL(br_rope_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(br_rope_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
     return 0;
 }

@@ -81,6 +81,16 @@ __device__ void stage_queries(const BrScoreParams& p, const BrPlanView& pv, int 
 
 // Dot products of one key row with the nq staged query vectors.  The head dim is a compile-time
 // constant so that the loop unrolls and every load of the key row is in flight before the first use.
+template <>
+struct Load8<_Float16> {
+    static __device__ inline void ld(const _Float16* p, float* x) {
+        uint4 u = *reinterpret_cast<const uint4*>(p);
+        const _Float16* h = reinterpret_cast<const _Float16*>(&u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = (float)h[i];
+    }
+};
+
 template <typename T, int D>
 __device__ inline void key_dots(const T* krow, const float* qs, int nq, float* s) {
 #pragma unroll
@@ -309,6 +319,10 @@ template <>
 __device__ inline void store_row_piece<__bf16>(__bf16* dst, const float* x, int n) {
     for (int i = 0; i < n; ++i) dst[i] = (__bf16)x[i];
 }
+template <>
+__device__ inline void store_row_piece<_Float16>(_Float16* dst, const float* x, int n) {
+    for (int i = 0; i < n; ++i) dst[i] = (_Float16)x[i];
+}
 
 // dk[key] = scale * sum over the kv head's query heads n and rows r of ds[n, r, key] * q[n, row_r].  One thread per key
 // slot, the whole row of D sums in its registers; the query vectors go through LDS sixteen (head, row) pairs at a time.
@@ -434,6 +448,18 @@ __global__ __launch_bounds__(256) void br_last_logits_bwd_dq_kernel(BrLogitsBwdP
 
 }  // namespace
 
+// Launch KERNEL<element type, head dim> for the dtype code (0 fp32, 1 bf16, 2 fp16) and D (64 or 128) in scope, 256
+// threads, with the parameter block p.
+#define BR_BY_TYPE_AND_DIM(KERNEL, GRID, LDS)                                                                   \
+    do {                                                                                                        \
+        if (dtype == 0 && D == 64) hipLaunchKernelGGL((KERNEL<float, 64>), GRID, dim3(256), LDS, stream, p);         \
+        else if (dtype == 0) hipLaunchKernelGGL((KERNEL<float, 128>), GRID, dim3(256), LDS, stream, p);              \
+        else if (dtype == 1 && D == 64) hipLaunchKernelGGL((KERNEL<__bf16, 64>), GRID, dim3(256), LDS, stream, p);   \
+        else if (dtype == 1) hipLaunchKernelGGL((KERNEL<__bf16, 128>), GRID, dim3(256), LDS, stream, p);             \
+        else if (D == 64) hipLaunchKernelGGL((KERNEL<_Float16, 64>), GRID, dim3(256), LDS, stream, p);               \
+        else hipLaunchKernelGGL((KERNEL<_Float16, 128>), GRID, dim3(256), LDS, stream, p);                           \
+    } while (0)
+
 // dtype: 0 fp32, 1 bf16
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
                          float* probs, const long long* sq, const long long* sk, int B, int Nq, int Nkv, int M, int H, int D,
@@ -448,14 +474,7 @@ int br_launch_doc_scores(const void* q, const void* k, const int* plan, const in
     const int chunks = (G + p.hc - 1) / p.hc;
     dim3 grid(M - 2, Nkv * chunks, B);
     size_t sh = (size_t)kQR * D * sizeof(float);
-    if (dtype == 0 && D == 64)
-        hipLaunchKernelGGL((br_doc_partial_kernel<float, 64>), grid, dim3(256), sh, stream, p);
-    else if (dtype == 0)
-        hipLaunchKernelGGL((br_doc_partial_kernel<float, 128>), grid, dim3(256), sh, stream, p);
-    else if (D == 64)
-        hipLaunchKernelGGL((br_doc_partial_kernel<__bf16, 64>), grid, dim3(256), sh, stream, p);
-    else
-        hipLaunchKernelGGL((br_doc_partial_kernel<__bf16, 128>), grid, dim3(256), sh, stream, p);
+    BR_BY_TYPE_AND_DIM(br_doc_partial_kernel, grid, sh);
     // the final kernel reuses hc as "the partials fit in LDS" flag
     size_t fin = (size_t)2 * Nq * R * sizeof(float);
     const size_t stage = (size_t)Nq * R * (M - 2) * 2 * sizeof(float);
@@ -479,14 +498,7 @@ int br_launch_last_logits(const void* q, const void* k, const int* plan, const i
     const int S = M * H;
     dim3 grid((S + 255) / 256, Nkv * chunks, B);
     size_t sh = (size_t)kQR * D * sizeof(float);
-    if (dtype == 0 && D == 64)
-        hipLaunchKernelGGL((br_last_logits_kernel<float, 64>), grid, dim3(256), sh, stream, p);
-    else if (dtype == 0)
-        hipLaunchKernelGGL((br_last_logits_kernel<float, 128>), grid, dim3(256), sh, stream, p);
-    else if (D == 64)
-        hipLaunchKernelGGL((br_last_logits_kernel<__bf16, 64>), grid, dim3(256), sh, stream, p);
-    else
-        hipLaunchKernelGGL((br_last_logits_kernel<__bf16, 128>), grid, dim3(256), sh, stream, p);
+    BR_BY_TYPE_AND_DIM(br_last_logits_kernel, grid, sh);
     return 0;
 }
 
@@ -522,18 +534,7 @@ int br_launch_last_logits_bwd(const float* ds, const void* q, const void* k, con
     p.B = B; p.Nq = Nq; p.Nkv = Nkv; p.M = M; p.H = H; p.D = D; p.R = R; p.T = T; p.scale = scale;
     const int S = M * H;
     dim3 gk((S + 255) / 256, Nkv, B), gq(Nq, B);
-    if (dtype == 0 && D == 64) {
-        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<float, 64>), gk, dim3(256), 0, stream, p);
-        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<float, 64>), gq, dim3(256), 0, stream, p);
-    } else if (dtype == 0) {
-        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<float, 128>), gk, dim3(256), 0, stream, p);
-        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<float, 128>), gq, dim3(256), 0, stream, p);
-    } else if (D == 64) {
-        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<__bf16, 64>), gk, dim3(256), 0, stream, p);
-        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<__bf16, 64>), gq, dim3(256), 0, stream, p);
-    } else {
-        hipLaunchKernelGGL((br_last_logits_bwd_dk_kernel<__bf16, 128>), gk, dim3(256), 0, stream, p);
-        hipLaunchKernelGGL((br_last_logits_bwd_dq_kernel<__bf16, 128>), gq, dim3(256), 0, stream, p);
-    }
+    BR_BY_TYPE_AND_DIM(br_last_logits_bwd_dk_kernel, gk, 0);
+    BR_BY_TYPE_AND_DIM(br_last_logits_bwd_dq_kernel, gq, 0);
     return 0;
 }

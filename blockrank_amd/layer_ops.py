@@ -14,7 +14,10 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib
-from .attention import _DTYPE_CODE, _stream_ptr
+from .attention import _DTYPE_CODE as _ALL_DTYPES, _stream_ptr
+
+# the norm / gate kernels are built for fp32 and bf16
+_DTYPE_CODE = {t: c for t, c in _ALL_DTYPES.items() if t in (torch.float32, torch.bfloat16)}
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:

@@ -76,7 +76,7 @@ def apply_rotary_pos_emb_fused(q: torch.Tensor, k: torch.Tensor, cos: torch.Tens
     kernel, which rotates every Q row in registers when it loads it - two passes over the largest tensor of the layer
     less.  Only for inference through that hook (bf16): any other consumer of the returned q would see it unrotated, so
     with gradients enabled, or dtypes the fused path does not take, both tensors are rotated here as usual."""
-    fused_ok = (q.dtype == torch.bfloat16 and q.is_cuda and cos.dim() == 3
+    fused_ok = (q.dtype in (torch.bfloat16, torch.float16) and q.is_cuda and cos.dim() == 3
                 and not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad)))
     if not fused_ok:
         return apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim)
@@ -101,7 +101,7 @@ def _rotate_impl(q, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, unsqu
         q = k
     assert unsqueeze_dim == 1, "only the (batch, heads, tokens, dim) convention of the decoder layers is supported"
     assert q.is_cuda and k.is_cuda and cos.is_cuda and sin.is_cuda, "the rotary embedding kernel needs device tensors"
-    assert q.dtype == k.dtype == cos.dtype == sin.dtype and q.dtype in _DTYPE_CODE, "q, k, cos and sin must share a dtype (bf16 or fp32)"
+    assert q.dtype == k.dtype == cos.dtype == sin.dtype and q.dtype in _DTYPE_CODE, "q, k, cos and sin must share a dtype (bf16, fp16 or fp32)"
     B, Nq, S, D = q.shape
     Nkv = k.shape[1]
     assert k.shape == (B, Nkv, S, D) and cos.shape[-2:] == (S, D) and sin.shape == cos.shape and cos.dim() == 3

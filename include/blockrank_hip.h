@@ -25,6 +25,7 @@ extern "C" {
 
 #define BR_DTYPE_F32 0
 #define BR_DTYPE_BF16 1
+#define BR_DTYPE_F16 2  /* forward attention, scores, rotary embedding; no backward, no fp8 variant, no log-sum-exp output */
 
 #define BR_OK 0
 #define BR_ERR_ARG 1      /* bad shape, dtype, alignment or null pointer (reference: AssertionError) */
@@ -83,7 +84,7 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D);
  *   multiple of 16 bytes, every base pointer 16-byte aligned.  out as the reference returns it,
  *   (B, S, Nq, D) contiguous, is strides {S*Nq*D, D, Nq*D}.
  *   Rows of real tokens receive the attention output; rows of padded slots are set to zero.
- *   D in {64, 128}; dtype BR_DTYPE_BF16 (bf16 MFMA, fp32 softmax/accumulate) or BR_DTYPE_F32. */
+ *   D in {64, 128}; dtype BR_DTYPE_BF16 or BR_DTYPE_F16 (MFMA of that type, fp32 softmax/accumulate) or BR_DTYPE_F32. */
 int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
                    int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
                    const int64_t* v_strides, const int64_t* out_strides, float scale, int dtype, void* workspace,
@@ -120,7 +121,7 @@ size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows);
  * This is the reference's "attention + s_last in one call" (blockrank_std_attention.py:623-645;
  * triton_blockrank_attention_forward with return_last_block_scores,
  * blockrank_triton_kernel_attention.py:858-881) without the second pass over K; the reference uses
- * score_rows = 16.  bf16 only (BR_DTYPE_F32 callers use br_doc_scores).  score_part needs no
+ * score_rows = 16.  bf16 and fp16 (BR_DTYPE_F32 callers use br_doc_scores).  score_part needs no
  * initialisation; it is consumed by br_doc_scores_from_partials with the same plan. */
 int br_prefill_fwd_scores(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
                           int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,

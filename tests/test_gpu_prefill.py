@@ -179,8 +179,8 @@ def test_error_behaviour():
         br.blockrank_attention_forward(None, q, k, v, torch.zeros(1, 1, 3, 8, device=DEV), 0.1)
     with pytest.raises(AssertionError):   # H != S // M
         br.blockrank_attention(q, k, v, torch.ones(1, 2, 8, dtype=torch.bool, device=DEV), 0.1)
-    with pytest.raises(NotImplementedError):
-        br.blockrank_attention(q.half(), k.half(), v.half(), lay.valid.to(DEV), 0.1)
+    with pytest.raises(NotImplementedError):   # a dtype without kernels
+        br.blockrank_attention(q.double(), k.double(), v.double(), lay.valid.to(DEV), 0.1)
     # gradients: bf16 attention has a backward; fp32 inputs and the fused score partials do not
     # (the reference's kernelised path refuses every backward, blockrank_triton_kernel_attention.py:759-761)
     with pytest.raises(NotImplementedError):
