@@ -60,12 +60,17 @@ int fail(int code, const char* fmt, ...) {
 
 // Head layout -> workgroup shape.  A workgroup carries NW row blocks of 32 query rows: Gw heads of
 // one kv head's group times tpb 32-token sub-blocks.
-bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW) {
+// ragged (the 16-bit MFMA forward kernels only): a group of 7 heads (Qwen2.5-7B's 28/4), which has no divisor but
+// itself, is cut into sub-groups of 4 + 3 (the spare wave of the second idles) instead of one workgroup of 7 waves:
+// two independent 4-wave workgroups per CU beat one wide one by a little more than the idle wave costs (measured 225
+// against 231 us at that shape).  Tokens per query tile are the same either way, so one plan serves both shapes.
+bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW, bool ragged = false) {
     if (Nq <= 0 || Nkv <= 0 || Nq % Nkv) return false;
     const int G = Nq / Nkv;
     int Gw = 1;
     for (int d = 1; d <= 8 && d <= G; ++d)
         if (G % d == 0) Gw = d;
+    if (ragged && Gw == 7) Gw = 4;
     int nw, tpb;
     switch (Gw) {
         case 1: nw = 4; tpb = 4; break;
@@ -77,7 +82,7 @@ bool make_geom(int Nq, int Nkv, BrGeom* g, int* NW) {
     g->G = G;
     g->Gw = Gw;
     g->tpb = tpb;
-    g->HGS = G / Gw;
+    g->HGS = (G + Gw - 1) / Gw;
     g->NHG = Nkv * g->HGS;
     *NW = nw;
     return true;
@@ -158,11 +163,14 @@ static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded
     if (!aligned16(plan)) return fail(BR_ERR_ARG, "plan buffer must be 16-byte aligned");
     const size_t need = br_plan_total_ints(B, M, H, T);
     if (plan_ints < need) return fail(BR_ERR_SPACE, "plan buffer holds %zu ints, %zu needed", plan_ints, need);
-    if ((long long)br_plan_max_items(B, M, H, T) * g.NHG >= (1 << 24))
+    BrGeom g16;
+    int nw16;
+    make_geom(Nq, Nkv, &g16, &nw16, true);                  // the shape the 16-bit forward kernels run in
+    if ((long long)br_plan_max_items(B, M, H, T) * (g16.NHG > g.NHG ? g16.NHG : g.NHG) >= (1 << 24))
         return fail(BR_ERR_ARG, "batch too large for one plan (B=%d, M=%d, H=%d)", B, M, H);
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
-    int par = n_cu * prefill_wgs_per_cu(nw) / g.NHG;       // workgroups of the prefill grid that share one head group's items
+    int par = n_cu * prefill_wgs_per_cu(nw16) / g16.NHG;    // workgroups of the prefill grid that share one head group's items
     par = par < 1 ? 1 : par;
     br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, par, plan, static_cast<hipStream_t>(stream));
     return check_launch("plan launch");
@@ -189,6 +197,10 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     int nw;
     if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || D <= 0) return 0;
     size_t rows = slots_total(B, g) * (size_t)nw * BR_RB;
+    // (the 16-bit kernels may cut a head group differently from the fp32 kernel: enough for either)
+    make_geom(Nq, Nkv, &g, &nw, true);
+    const size_t rows16 = slots_total(B, g) * (size_t)nw * BR_RB;
+    rows = rows16 > rows ? rows16 : rows;
     return rows * (size_t)(D + 2) * sizeof(float);
 }
 
@@ -279,7 +291,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         return rc;
     BrGeom g;
     int nw;
-    make_geom(Nq, Nkv, &g, &nw);
+    make_geom(Nq, Nkv, &g, &nw, dtype != BR_DTYPE_F32);
     if (fp8_tokens > 0 && (dtype != BR_DTYPE_BF16 || D != 128))
         return fail(BR_ERR_ARG, "the fp8 Q K^T variant takes bf16 inputs with head dim 128");
     const size_t need = fp8_tokens > 0 ? br_prefill_fp8qk_workspace_bytes(B, Nq, Nkv, D, M, fp8_tokens) : br_prefill_workspace_bytes(B, Nq, Nkv, D);

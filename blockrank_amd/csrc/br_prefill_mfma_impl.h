@@ -552,10 +552,15 @@ struct Prefill {
         const int b = it.b, m = it.m;
         const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
         const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
-        const int head = kvh * ge.G + hsub * ge.Gw + g;
+        // (a kv head's group need not be a multiple of Gw: the last sub-group then has waves without a head, which
+        // stay with the workgroup - barriers, DMA - and neither load rows nor store anything)
+        const int hpos = hsub * ge.Gw + g;
+        const bool head_ok = hpos < ge.G;
+        const int head = kvh * ge.G + (head_ok ? hpos : ge.G - 1);
         const int len_m = it.len_m;
+        const int len_w = head_ok ? len_m : 0;             // the block's length as far as this wave's rows go
         const int row0 = it.t0 + sub * BR_RB;              // first query row of this wave, valid-relative
-        const bool rb_active = row0 < len_m;
+        const bool rb_active = row0 < len_w;
         const int self_end = it.t0 + T < len_m ? it.t0 + T : len_m;
         const int qtok0 = it.tok_m;                        // token index of the block's first real token
         const unsigned smem_lds = lds_addr_of(smem);
@@ -780,7 +785,7 @@ struct Prefill {
                 const float tot = psum + __shfl_xor(psum, 32);
                 const int ln_l = lane_l & 31;
                 const int r16 = it.start_m + row0 + ln_l - (p.H - p.score_R);
-                if (lane_l < 32 && r16 >= 0 && row0 + ln_l < len_m) {
+                if (lane_l < 32 && r16 >= 0 && row0 + ln_l < len_w) {
                     float2 ms = make_float2(m_run == -INFINITY ? 0.f : m_run, tot);
                     *reinterpret_cast<float2*>(p.score_part + ((((long long)b * p.Nq + head) * p.score_R + r16) * pv.tps + c_f) * 2) = ms;
                 }
@@ -802,7 +807,7 @@ struct Prefill {
         const float l_tot = l_run + __shfl_xor(l_run, 32);       // exact sum: log-sum-exp
         const float lt_tot = lt_run + __shfl_xor(lt_run, 32);    // sum of the rounded probabilities: normalises the output
         if (it.slot >= 0) {
-            if (row0 + ln < len_m) {
+            if (row0 + ln < len_w) {
                 const long long slot = ((long long)b * BR_SLOTS_PER_SEQ + it.slot) * ge.NHG + hg;
                 const long long prow = slot * (NW * BR_RB) + wave * BR_RB + ln;
                 float* po = p.part_o + prow * D;
@@ -823,7 +828,7 @@ struct Prefill {
             // through LDS so that every output row is written as full 16-byte pieces
             BR_E16* Es = reinterpret_cast<BR_E16*>(smem + wave * SM::eBytesPerWave);
             const float inv = lt_tot > 0.f ? __builtin_amdgcn_rcpf(lt_tot) : 0.f;
-            if (p.lse != nullptr && lane_e < 32 && row0 + lane_e < len_m)
+            if (p.lse != nullptr && lane_e < 32 && row0 + lane_e < len_w)
                 p.lse[(long long)b * p.lse_b + (long long)head * p.lse_h + qtok0 + row0 + lane_e] = m_run + __builtin_amdgcn_logf(l_tot);
             if (rb_active) {
 #pragma unroll
@@ -865,7 +870,8 @@ struct Prefill {
         // document and head group; a packed layout has no padded slots).  The prefix's and the query block's
         // are left to the finish kernel: their items are the ones the others wait for.
         if (it.t0 == 0 && m > 0 && m < p.M - 1 && padded_layout)
-            zero_padded_rows<D>(p, b, kvh * ge.G + hsub * ge.Gw, ge.Gw, it.tok_m - it.start_m, it.start_m, len_m, tid, NW * 64);
+            zero_padded_rows<D>(p, b, kvh * ge.G + hsub * ge.Gw, ge.G - hsub * ge.Gw < ge.Gw ? ge.G - hsub * ge.Gw : ge.Gw,
+                                it.tok_m - it.start_m, it.start_m, len_m, tid, NW * 64);
     }
 };
 
@@ -970,7 +976,7 @@ __global__ __launch_bounds__(THREADS) void br_finish_kernel(BrPrefillParams p, i
         const int qtok0 = pv.tok[c.b * p.M + m];
         const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
         const int row = c.t0 + sub * BR_RB + rloc;
-        if (row >= len_m) continue;
+        if (row >= len_m || hsub * ge.Gw + g >= ge.G) continue;     // (the second: a wave without a head, ragged group)
         const int head = kvh * ge.G + hsub * ge.Gw + g;
         const long long slot0 = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0) * ge.NHG + hg;
         const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
