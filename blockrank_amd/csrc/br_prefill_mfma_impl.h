@@ -550,8 +550,10 @@ struct Prefill {
         const BrGeom& ge = p.geom;
         const int T = ge.tpb * BR_RB;
         const int b = it.b, m = it.m;
-        const int kvh = hg / ge.HGS, hsub = hg - kvh * ge.HGS;
-        const int g = wave / ge.tpb, sub = wave - g * ge.tpb;
+        // (tpb is 1, 2 or 4 and a kv head usually has one sub-group: no integer divisions on the way to the first load)
+        const int kvh = ge.HGS == 1 ? hg : hg / ge.HGS, hsub = hg - kvh * ge.HGS;
+        const int tsh = ge.tpb == 1 ? 0 : (ge.tpb == 2 ? 1 : 2);
+        const int g = wave >> tsh, sub = wave & (ge.tpb - 1);
         // (a kv head's group need not be a multiple of Gw: the last sub-group then has waves without a head, which
         // stay with the workgroup - barriers, DMA - and neither load rows nor store anything)
         const int hpos = hsub * ge.Gw + g;
