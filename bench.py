@@ -56,6 +56,7 @@ def workloads():
         # Qwen2.5-7B head layout and a long-tailed document length distribution (bf16; --qk-fp8 computes Q K^T in fp8)
         "cfg5shape": dict(desc="Qwen2.5-7B attention shapes, B=4, 28q/4kv heads, D=128, 32-token prefix + 50 lognormal docs + 24-token query, bf16",
                           layout=lambda: synthetic.lognormal_layout(4, 32, 50, 120, 0.6, 16, 512, 24, seed=0), Nq=28, Nkv=4, D=128, hidden=3584, dtype=torch.bfloat16),
+        "cfg2d64": dict(desc="cfg2 layout with head dim 64", layout=lambda: synthetic.uniform_layout(4, 64, 20, 160, 32), Nq=32, Nkv=8, D=64, hidden=None, dtype=torch.bfloat16),
         "cfg2_b1": dict(desc="cfg2 with B=1", layout=lambda: synthetic.uniform_layout(1, 64, 20, 160, 32), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
         "cfg2_b16": dict(desc="cfg2 with B=16", layout=lambda: synthetic.uniform_layout(16, 64, 20, 160, 32), Nq=32, Nkv=8, D=128, hidden=4096, dtype=torch.bfloat16),
         # one long causal block per sequence: many key tiles per work item (steady-state tile throughput)
