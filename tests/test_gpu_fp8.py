@@ -5,8 +5,8 @@ are read from - are computed on the bf16 Q and K.  Two checks:
   * against the oracle fed with the same quantised Q and K (oracle.quantize_fp8_e4m3) for the prefix and
     document rows and with the unquantised ones for the query block: the kernel's own arithmetic, to the
     usual bf16 bar (outputs 2e-2 max-abs, scores 1e-3 relative);
-  * against the unquantised fp32 oracle, the variant as a whole, at what config 5 states: every score within
-    5e-3 relative, identical top-10."""
+  * against the unquantised fp32 oracle, the variant as a whole, at the bound that benchmark configuration states:
+    every score within 5e-3 relative, identical top-10."""
 import numpy as np
 import pytest
 import torch
