@@ -385,6 +385,7 @@ def blockrank_attention(
             part = torch.empty(max(opt.score_part_bytes // 4, 4), dtype=torch.float32, device=dev)
             opt.score_part = part.data_ptr()
         if rank_rows is not None:
+            assert M >= 3, "per-document scores need at least one document block"
             assert rank_rows.shape[0] == B and rank_rows.dim() == 2, "rank_rows must be (B, R)"
             rr = rank_rows.to(device=dev, dtype=torch.int32).contiguous()
             scores = torch.empty((B, M - 2), dtype=torch.float32, device=dev)
