@@ -14,7 +14,7 @@
 #define BR_RB 32              // query rows per wave (one 32x32 MFMA row block)
 #define BR_SLOTS_PER_SEQ 32   // split-KV partial slots available to one sequence's query block
 #ifndef BR_MIN_CHUNK
-#define BR_MIN_CHUNK 8        // a split of the query block's key walk covers at least this many tiles
+#define BR_MIN_CHUNK 4        // a split of the query block's key walk covers at least this many tiles
 #endif
 
 // Plan buffer (int32):

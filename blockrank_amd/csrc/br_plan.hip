@@ -158,25 +158,33 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
 
     // Length of a split of the query block's key walk.  The walk is cut so that the batch has enough items to fill
     // the grid, and no further: every split costs a set-up, an epilogue and a set of partials to write and merge,
-    // while a split as long as the whole kernel's share per workgroup still ends with the others because the split
-    // items are handed out first.  So: about the estimated work per workgroup (all items' key tiles plus their
-    // constant, over the workgroups that run side by side), and at least BR_MIN_CHUNK.
-    long long w_all = 0;
+    // while a long split still ends with the others because the split items are handed out first.  So: the estimated
+    // work per workgroup (all items' key tiles plus their constant, over the workgroups that run side by side) less
+    // one ordinary item - the workgroup that takes a split still has to fit one of those before the kernel ends, which
+    // is what decides at a batch of one - and at least BR_MIN_CHUNK.
+    long long w_all = 0, w_ord = 0;
+    int n_ord = 0;
     for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
         const int p = p0 + tid;
-        int w = 0;
+        int w = 0, nq = 0;
+        bool last = false;
         if (p < BM) {
             const int b = p / M, m = p - b * M;
             const int L = len[p];
-            const int nq = ceil_div(L, T);
-            const int np = m == M - 1 ? (M > 1 ? prev_tiles[b] : 0) : (br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0);
+            nq = ceil_div(L, T);
+            last = m == M - 1;
+            const int np = last ? (M > 1 ? prev_tiles[b] : 0) : (br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0);
             for (int tt = 0; tt < nq; ++tt) w += item_weight(np, tt, L);
         }
         int tot;
         block_exclusive_scan(w, sh, &tot);
         w_all += tot;
+        block_exclusive_scan(last ? 0 : w, sh, &tot);
+        w_ord += tot;
+        block_exclusive_scan(last ? 0 : nq, sh, &tot);
+        n_ord += tot;
     }
-    int chunk = (int)(w_all / (par > 0 ? par : 1));
+    int chunk = (int)(w_all / (par > 0 ? par : 1)) - (n_ord > 0 ? (int)(w_ord / n_ord) : 0);
     chunk = chunk < BR_MIN_CHUNK ? BR_MIN_CHUNK : chunk;
 
     struct Counts {
