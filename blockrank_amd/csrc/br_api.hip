@@ -12,9 +12,9 @@
 void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int* plan,
                     hipStream_t stream);
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
+                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank, int wave_rows);
 int br_launch_prefill_f16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                          hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
+                          hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank, int wave_rows);
 int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                            hipEvent_t ev_start, hipEvent_t ev_stop);
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
@@ -362,8 +362,10 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         p.qk_scales = scales;
         lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp);
     } else {
-        lrc = dtype == BR_DTYPE_BF16  ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
-              : dtype == BR_DTYPE_F16 ? br_launch_prefill_f16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
+        const char* wr_env = getenv("BLOCKRANK_AMD_WAVE_ROWS");
+        const int wave_rows = wr_env ? atoi(wr_env) : 32;
+        lrc = dtype == BR_DTYPE_BF16  ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp, wave_rows)
+              : dtype == BR_DTYPE_F16 ? br_launch_prefill_f16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp, wave_rows)
                                       : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s, e0, e1);
     }
     if (lrc) return fail(BR_ERR_ARG, "no kernel for head dim %d with %d query heads per kv head", D, g.G);

@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void br_quant_pass_kernel(BrQuantParams p) {
 
 template <int D, int NW>
 void launch8(const BrPrefillParams& p, int grid, hipStream_t stream) {
-    hipLaunchKernelGGL((br_prefill_mfma_kernel<D, NW, true>), dim3(grid), dim3(NW * 64), 0, stream, p);
+    hipLaunchKernelGGL((br_prefill_mfma_kernel<D, NW, true, true, false>), dim3(grid), dim3(NW * 64), 0, stream, p);
 }
 
 }  // namespace

@@ -289,7 +289,10 @@ typedef long k8x8;   // eight fp8 values: one MFMA operand of v_mfma_f32_32x32x1
 template <bool F8> struct QKFrag { typedef e16x8 type; };
 template <> struct QKFrag<true> { typedef k8x8 type; };
 
-template <int D, int NW, bool F8>
+// SC: the instance that can leave score partials and the log-sum-exp (exact probability sums); ROPE: the instance
+// that rotates the Q rows it loads.  An instance without them carries none of their registers, scalars or code
+// (the plain layers of a ranking forward use neither).
+template <int D, int NW, bool F8, bool SC = true, bool ROPE = true>
 struct Prefill {
     using SM = Smem<D, F8>;
     using Frag = typename QKFrag<F8>::type;                // K and Q operand of one 16-dim chunk
@@ -314,6 +317,14 @@ struct Prefill {
     // line and the shift that separates them is 1.
     static constexpr int VSW = CPR == 16 ? 2 : 1;
     static constexpr int STEP_ROWSK = NW * 64 / CPRK;      // ... K pieces
+    // K swizzle: LDS piece = global piece ^ (row & KSW).  An operand read takes one 16-byte piece of each of 32 rows;
+    // the 16 lanes that go through the banks together (16 x 16 bytes = one pass over all 64 banks) must hit 16
+    // different pieces, so with 16 pieces per row the whole row index's low four bits take part (with 8 pieces per
+    // row two rows share a 256-byte bank line and three bits do).
+#ifndef BR_K_SWIZZLE_MASK
+#define BR_K_SWIZZLE_MASK 15
+#endif
+    static constexpr int KSW = CPRK >= 16 ? BR_K_SWIZZLE_MASK : (CPRK < 8 ? CPRK - 1 : 7);
     struct Lane {
         int koff[JOK], voff[JO];   // global byte offsets inside a tile of this lane's DMA pieces
         int krd;                   // LDS byte offset of the K operand read of chunk 0; chunk c is krd ^ (c << (F8 ? 4 : 5))
@@ -327,7 +338,7 @@ struct Prefill {
             const int slot = (wave + NW * j) * 64 + lane;
             const int prow = slot / CPRK, cp = slot - prow * CPRK;
             const int kkey = (prow & 32) | swap23(prow & 31);
-            L.koff[j] = kkey * (F8 ? D : (int)p.k32_t * 2) + ((cp ^ (prow & (CPRK < 8 ? CPRK - 1 : 7))) << 4);
+            L.koff[j] = kkey * (F8 ? D : (int)p.k32_t * 2) + ((cp ^ (prow & KSW)) << 4);
         }
 #pragma unroll
         for (int j = 0; j < JO; ++j) {
@@ -336,8 +347,8 @@ struct Prefill {
             L.voff[j] = prow * (int)p.v32_t * 2 + ((cp ^ ((prow & 3) << VSW)) << 4);
         }
         const int ln = lane & 31, lh = lane >> 5;
-        if (F8) L.krd = ln * SM::rowKB + (((ln & (CPRK < 8 ? CPRK - 1 : 7))) << 4) + lh * 8;   // 8 bytes: dims 16c + 8lh .. +7
-        else L.krd = ln * SM::rowKB + ((lh ^ (ln & 7)) << 4);
+        if (F8) L.krd = ln * SM::rowKB + ((ln & KSW) << 4) + lh * 8;   // 8 bytes: dims 16c + 8lh .. +7
+        else L.krd = ln * SM::rowKB + ((lh ^ (ln & KSW)) << 4);
         // transposing read: within a group of 16 lanes, lane s points at key (s >> 2), dims 4 * (s & 3)
         const int s = lane & 15, ln_hi = (lane >> 4) & 1;
 #pragma unroll
@@ -589,8 +600,11 @@ struct Prefill {
         const int2* tiles_b = pv.tiles + (size_t)b * pv.tps;
         const bool table = it.pe > 1;
         // only query-block items of a sequence with documents emit score partials, for document tiles
-        const bool emit_scores = p.score_part != nullptr && table && m == p.M - 1;
-        const bool exact = emit_scores || p.lse != nullptr;
+        bool emit_scores = false, exact = false;
+        if constexpr (SC) {
+            emit_scores = p.score_part != nullptr && table && m == p.M - 1;
+            exact = emit_scores || p.lse != nullptr;
+        }
         const int first_doc_tile = (it.len0 + BR_BN - 1) / BR_BN;
         const int nprev = it.nprev;
         const int f_end = it.ntiles > 0x3fffffff ? 0x7fffffff : it.f_lo + it.ntiles;
@@ -609,9 +623,11 @@ struct Prefill {
         Frag qf[D / 16];
         u32x4 qraw[F8 ? D / 16 : 1];       // fp8: the bf16 rows as loaded, converted once they have arrived
         // rotary embedding applied here: the row's cos / sin values for the lane's dims (both halves of the tables)
-        constexpr int NRC = F8 ? 1 : D / 32;
-        e16x8 rcos[2][NRC], rsin[2][NRC];
-        const bool rope = !F8 && p.rope_cos != nullptr && rb_active;
+        constexpr bool DO_ROPE = ROPE && !F8;
+        constexpr int NRC = DO_ROPE ? D / 32 : 1;
+        e16x8 rcos[2][DO_ROPE ? NRC : 0], rsin[2][DO_ROPE ? NRC : 0];
+        bool rope = false;
+        if constexpr (DO_ROPE) rope = p.rope_cos != nullptr && rb_active;
         {
             const char* qrow = reinterpret_cast<const char*>(p.q) +
                                ((unsigned long long)p.q32_b * (unsigned)b + (unsigned long long)p.q32_h * (unsigned)head +
@@ -633,7 +649,7 @@ struct Prefill {
                     else qf[c] = as_e16x8(uint4{0u, 0u, 0u, 0u});
                 }
             }
-            if constexpr (!F8) {
+            if constexpr (DO_ROPE) {
                 if (rope) {
                     const long long tbl = ((long long)p.rope_b * b + (long long)p.rope_t * (qtok0 + row0 + (ln < last ? ln : last))) * 2 + lh * 16;
                     const char* crow = reinterpret_cast<const char*>(p.rope_cos) + tbl;
@@ -709,7 +725,7 @@ struct Prefill {
 #pragma unroll
             for (int c = 0; c < D / 16; ++c) qf[c] = quantize_q8(qraw[c], q_inv);
         }
-        if constexpr (!F8) {
+        if constexpr (DO_ROPE) {
             // out = x cos + rotate_half(x) sin: dim d < D/2 pairs with d + D/2, which the same lane holds D/32 chunks
             // further on; fp32 arithmetic, one rounding (what the stand-alone rotary kernel computes)
             if (rope) {
@@ -767,14 +783,19 @@ struct Prefill {
             if (nkb > 0) {
                 const int lim_causal = c_self ? row0 + ln - key0 + 1 : BR_BN;   // keys [0, lim) visible
                 const int lim = v_nvalid < lim_causal ? v_nvalid : lim_causal;
-                int v_exact = exact ? 1 : 0;                 // (a per-lane value, like the tile quantities above)
-                asm volatile("" : "+v"(v_exact));
-                if (v_exact != 0) {
-                    if (nkb == 2 && !need_mask) compute_tile<2, false, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, 0, lh, psum);
-                    else if (nkb == 2) compute_tile<2, true, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
-                    else if (need_mask) compute_tile<1, true, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
-                    else compute_tile<1, false, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
-                } else {
+                bool done = false;
+                if constexpr (SC) {
+                    int v_exact = exact ? 1 : 0;             // (a per-lane value, like the tile quantities above)
+                    asm volatile("" : "+v"(v_exact));
+                    if (v_exact != 0) {
+                        if (nkb == 2 && !need_mask) compute_tile<2, false, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, 0, lh, psum);
+                        else if (nkb == 2) compute_tile<2, true, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                        else if (need_mask) compute_tile<1, true, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                        else compute_tile<1, false, true>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
+                        done = true;
+                    }
+                }
+                if (!done) {
                     if (nkb == 2 && !need_mask) compute_tile<2, false, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, 0, lh, psum);
                     else if (nkb == 2) compute_tile<2, true, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
                     else if (need_mask) compute_tile<1, true, false>(stage, L, qf, o, m_run, l_run, lt_run, sc2, lim, lh, psum);
@@ -783,7 +804,7 @@ struct Prefill {
             }
             // Score partials: this tile's probability mass (against the running max) for the query block's
             // last rows, per head - everything the per-document scores need, with no second pass over K.
-            if (emit_scores && nkb > 0 && !c_self && c_f >= first_doc_tile) {
+            if (SC && emit_scores && nkb > 0 && !c_self && c_f >= first_doc_tile) {
                 const float tot = psum + __shfl_xor(psum, 32);
                 const int ln_l = lane_l & 31;
                 const int r16 = it.start_m + row0 + ln_l - (p.H - p.score_R);
@@ -830,7 +851,7 @@ struct Prefill {
             // through LDS so that every output row is written as full 16-byte pieces
             BR_E16* Es = reinterpret_cast<BR_E16*>(smem + wave * SM::eBytesPerWave);
             const float inv = lt_tot > 0.f ? __builtin_amdgcn_rcpf(lt_tot) : 0.f;
-            if (p.lse != nullptr && lane_e < 32 && row0 + lane_e < len_w)
+            if (SC && p.lse != nullptr && lane_e < 32 && row0 + lane_e < len_w)
                 p.lse[(long long)b * p.lse_b + (long long)head * p.lse_h + qtok0 + row0 + lane_e] = m_run + __builtin_amdgcn_logf(l_tot);
             if (rb_active) {
 #pragma unroll
@@ -877,14 +898,14 @@ struct Prefill {
     }
 };
 
-template <int D, int NW, bool F8>
+template <int D, int NW, bool F8, bool SC, bool ROPE>
 __global__ __launch_bounds__(NW * 64, 2) void br_prefill_mfma_kernel(BrPrefillParams p) {
     // one LDS object, so that it starts at LDS address 0 and every DMA target stays below 64 KiB;
     // the two descriptor mailboxes sit behind the tile stages
     __shared__ __attribute__((aligned(1024))) char smem[Smem<D, F8>::total(NW) + 2 * sizeof(BrDescMail)];
     BrDescMail* mail = reinterpret_cast<BrDescMail*>(smem + Smem<D, F8>::total(NW));
-    using PF = Prefill<D, NW, F8>;
-    using PF16 = Prefill<D, NW, false>;
+    using PF = Prefill<D, NW, F8, SC, ROPE>;
+    using PF16 = Prefill<D, NW, false, SC, ROPE>;
     const int NHG = p.geom.NHG;
     const BrPlanView pv = br_plan_view(p.plan, p.B, p.M, p.H, p.geom.tpb * BR_RB);
     int* hdr = const_cast<int*>(p.plan);
