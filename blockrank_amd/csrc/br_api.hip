@@ -9,8 +9,8 @@
 #include "br_common.h"
 #include "br_score_tiles.h"
 
-void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int* plan,
-                    hipStream_t stream);
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int pool,
+                    int* plan, hipStream_t stream);
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                            hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank, int wave_rows);
 int br_launch_prefill_f16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
@@ -43,7 +43,7 @@ void br_launch_silu_mul(const void* gate, const void* up, void* out, long long n
 // Split-KV partials of br_prefill_fwd_noalloc: device memory that belongs to the library, one copy on every GPU
 // the library runs on, held until the process ends.  In host code this name is only a handle for
 // hipGetSymbolAddress: the address the kernels get is the one that call returns for the current device.
-#define BR_NOALLOC_SCRATCH_BYTES ((size_t)80 << 20)
+#define BR_NOALLOC_SCRATCH_BYTES ((size_t)32 << 20)
 static __device__ __align__(256) unsigned char scratch[BR_NOALLOC_SCRATCH_BYTES];
 
 namespace {
@@ -128,7 +128,17 @@ int check_strides(const char* name, const int64_t* s, int dtype) {
     return BR_OK;
 }
 
-size_t slots_total(int B, const BrGeom& g) { return (size_t)B * BR_SLOTS_PER_SEQ * g.NHG; }
+// Workgroups of the 16-bit prefill grid that share one head group's items: what the plan balances the split of the
+// query blocks' walks against, and what sizes the pool of split-KV partial slots.
+int prefill_par(int Nq, int Nkv, int n_cu) {
+    BrGeom g16;
+    int nw16;
+    if (!make_geom(Nq, Nkv, &g16, &nw16, true)) return 1;
+    const int par = n_cu * prefill_wgs_per_cu(nw16) / g16.NHG;
+    return par < 1 ? 1 : par;
+}
+
+size_t slots_total(int pool, const BrGeom& g) { return (size_t)pool * g.NHG; }
 
 }  // namespace
 
@@ -152,6 +162,24 @@ size_t br_plan_ints(int B, int M, int H, int Nq, int Nkv) {
     return br_plan_total_ints(B, M, H, br_tokens_per_tile(g));
 }
 
+// Address of this device's copy of the scratch array, looked up once per device (with that device current).
+static int noalloc_scratch(void** out) {
+    constexpr int kMaxDev = 64;
+    static std::atomic<void*> ptrs[kMaxDev];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(BR_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDev) return fail(BR_ERR_HIP, "device index %d out of range", dev);
+    void* ptr = ptrs[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) return fail(BR_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        ptrs[dev].store(ptr, std::memory_order_release);     // every thread gets the same address for a device
+    }
+    *out = ptr;
+    return BR_OK;
+}
+
 static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded, int packed, int B, int M, int H, int Nq, int Nkv,
                       int32_t* plan, size_t plan_ints, void* stream) {
     if (B <= 0 || M <= 0 || H <= 0) return fail(BR_ERR_ARG, "B, M and H must be positive (got %d, %d, %d)", B, M, H);
@@ -170,9 +198,13 @@ static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded
         return fail(BR_ERR_ARG, "batch too large for one plan (B=%d, M=%d, H=%d)", B, M, H);
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
-    int par = n_cu * prefill_wgs_per_cu(nw16) / g16.NHG;    // workgroups of the prefill grid that share one head group's items
-    par = par < 1 ? 1 : par;
-    br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, par, plan, static_cast<hipStream_t>(stream));
+    // (the set-up call of every request: look the no-alloc entry's scratch array up here, so that the entry itself
+    // never has to - the first lookup on a device makes the runtime load the code object)
+    void* scratch_ptr = nullptr;
+    int src = noalloc_scratch(&scratch_ptr);
+    if (src) return src;
+    const int par = prefill_par(Nq, Nkv, n_cu);
+    br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, par, br_split_pool(par), plan, static_cast<hipStream_t>(stream));
     return check_launch("plan launch");
 }
 
@@ -196,10 +228,13 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     BrGeom g;
     int nw;
     if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || D <= 0) return 0;
-    size_t rows = slots_total(B, g) * (size_t)nw * BR_RB;
+    const int n_cu = n_compute_units();
+    if (n_cu <= 0) return 0;
+    const int pool = br_split_pool(prefill_par(Nq, Nkv, n_cu));
+    size_t rows = slots_total(pool, g) * (size_t)nw * BR_RB;
     // (the 16-bit kernels may cut a head group differently from the fp32 kernel: enough for either)
     make_geom(Nq, Nkv, &g, &nw, true);
-    const size_t rows16 = slots_total(B, g) * (size_t)nw * BR_RB;
+    const size_t rows16 = slots_total(pool, g) * (size_t)nw * BR_RB;
     rows = rows16 > rows ? rows16 : rows;
     return rows * (size_t)(D + 2) * sizeof(float);
 }
@@ -301,7 +336,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
 
     BrPrefillParams p;
     p.q = q; p.k = k; p.v = v; p.out = out; p.plan = plan;
-    const size_t rows = slots_total(B, g) * (size_t)nw * BR_RB;
+    const size_t rows = slots_total(br_split_pool(prefill_par(Nq, Nkv, n_cu)), g) * (size_t)nw * BR_RB;
     p.part_o = static_cast<float*>(workspace);
     p.part_ml = p.part_o + rows * D;
     p.sq_b = q_strides[0]; p.sq_h = q_strides[1]; p.sq_t = q_strides[2];
@@ -389,30 +424,13 @@ int br_prefill_fwd(const void* q, const void* k, const void* v, void* out, const
 
 size_t br_prefill_noalloc_max_workspace_bytes(void) { return BR_NOALLOC_SCRATCH_BYTES; }
 
-// Address of this device's copy of the scratch array, looked up once per device (with that device current).
-static int noalloc_scratch(void** out) {
-    constexpr int kMaxDev = 64;
-    static std::atomic<void*> ptrs[kMaxDev];
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return fail(BR_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
-    if (dev < 0 || dev >= kMaxDev) return fail(BR_ERR_HIP, "device index %d out of range", dev);
-    void* ptr = ptrs[dev].load(std::memory_order_acquire);
-    if (!ptr) {
-        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-        if (e != hipSuccess || !ptr) return fail(BR_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
-        ptrs[dev].store(ptr, std::memory_order_release);     // every thread gets the same address for a device
-    }
-    *out = ptr;
-    return BR_OK;
-}
-
 int br_prefill_fwd_noalloc(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq, int Nkv,
                            int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                            const int64_t* out_strides, float scale, int dtype, void* stream) {
     int rc = check_common(B, Nq, Nkv, M, H, D, dtype);
     if (rc) return rc;
     const size_t need = br_prefill_workspace_bytes(B, Nq, Nkv, D);
+    if (need == 0) return fail(BR_ERR_HIP, "no HIP device");
     if (need > BR_NOALLOC_SCRATCH_BYTES)
         return fail(BR_ERR_SPACE, "br_prefill_fwd_noalloc: B=%d with %d/%d heads of dim %d needs %zu bytes of partials, the built-in scratch holds %zu; "
                                   "use br_prefill_fwd with a workspace, or a smaller batch", B, Nq, Nkv, D, need, (size_t)BR_NOALLOC_SCRATCH_BYTES);

@@ -12,7 +12,11 @@
 
 #define BR_BN 64              // keys per key/value tile
 #define BR_RB 32              // query rows per wave (one 32x32 MFMA row block)
-#define BR_SLOTS_PER_SEQ 32   // split-KV partial slots available to one sequence's query block
+// Split-KV partial slots of the query blocks' key walks: one pool for the whole batch, handed out by the plan in
+// item order.  Splitting exists to give every workgroup of the grid something to do, so the pool is a fraction of
+// the workgroups that share a head group's items (par) and does not grow with the batch: br_split_pool(par) slots,
+// at most BR_SPLIT_POOL_MAX.  The plan lengthens the splits until the batch fits the pool.
+#define BR_SPLIT_POOL_MAX 160
 #ifndef BR_MIN_CHUNK
 #define BR_MIN_CHUNK 4        // a split of the query block's key walk covers at least this many tiles
 #endif
@@ -41,6 +45,8 @@ enum BrPlanHeader {
     BR_PH_MAX_ITEMS = 5,
     BR_PH_MAX_COMB = 6,
     BR_PH_T = 7,          // tokens per query tile the plan was built for
+    BR_PH_POOL = 26,      // split-KV slots the plan was built for
+    BR_PH_NSLOTS = 27,    // ... and how many of them it uses
     BR_PH_QCOUNT = 8,     // [9] items in each queue
     BR_PH_QOFF = 17,      // [9] index of each queue's first item
     // second cache line: everything the running kernels update
@@ -53,7 +59,7 @@ enum BrPlanHeader {
 // (the sequence's first nprev tile descriptors), then the tiles of its own block up to the diagonal.
 // f_lo is the first tile of the range in that order, ntiles how many to process (INT_MAX = to the
 // end).  slot < 0: the item owns its rows and writes the final output; slot >= 0: it writes an
-// unnormalised partial into that slot.  The item also carries what the kernel would otherwise have
+// unnormalised partial into that slot of the batch's pool.  The item also carries what the kernel would otherwise have
 // to look up before it can issue its first load: the block's own span and the prefix block's span.
 struct BrItem {
     int b, m, t0, f_lo, nprev, ntiles, slot, pe;
@@ -84,12 +90,17 @@ __host__ __device__ inline size_t br_plan_off_start() { return BR_PLAN_HDR; }
 __host__ __device__ inline size_t br_plan_off_len(int B, int M) { return BR_PLAN_HDR + (size_t)B * M; }
 __host__ __device__ inline size_t br_plan_off_tok(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M; }
 __host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLAN_HDR + 3 * (size_t)B * M; }
+__host__ __device__ inline int br_split_pool(int par) {
+    const int n = par / 4 + 2;
+    return n > BR_SPLIT_POOL_MAX ? BR_SPLIT_POOL_MAX : n;
+}
 __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
     int qt = (H + T - 1) / T;
-    int last = qt > BR_SLOTS_PER_SEQ ? qt : BR_SLOTS_PER_SEQ;
-    return B * ((M > 1 ? (M - 1) * qt : 0) + last);
+    // every query tile of every block once, plus one more item per slot a split query tile takes
+    return B * (M > 1 ? M : 1) * qt + BR_SPLIT_POOL_MAX;
 }
-__host__ __device__ inline int br_plan_max_comb(int B) { return B * (BR_SLOTS_PER_SEQ / 2); }
+// (a split query tile takes at least two slots)
+__host__ __device__ inline int br_plan_max_comb(int B) { return BR_SPLIT_POOL_MAX / 2; }
 __host__ __device__ inline int br_plan_tps(int M, int H) { return (M > 1 ? M - 1 : 0) * ((H + BR_BN - 1) / BR_BN); }
 __host__ __device__ inline size_t br_plan_off_tbase(int B, int M) { return BR_PLAN_HDR + 3 * (size_t)B * M + (size_t)B; }
 __host__ __device__ inline size_t br_plan_off_tiles(int B, int M) { return (br_plan_off_tbase(B, M) + (size_t)B * M + 1) & ~(size_t)1; }

@@ -10,9 +10,6 @@
 namespace {
 
 constexpr int kPlanThreads = 1024;
-#ifndef BR_TILE_ORDER_DESC
-#define BR_TILE_ORDER_DESC 1
-#endif
 
 // One wave per block: count real tokens, find the first and the last.  len is written negated
 // (-1 - count) when the real tokens are not one contiguous span; the plan kernel repairs the sign
@@ -69,16 +66,15 @@ __device__ int block_exclusive_scan(int x, int* sh, int* total) {
     return base + incl - x;
 }
 
-// Split count for a query tile of the query block: enough splits that each covers about ``chunk`` key tiles,
-// limited so that all tiles of the block fit the sequence's slot budget.
-__device__ inline int splits_for(int ntiles, int ns_cap, int chunk) {
-    int ns = ceil_div(ntiles, chunk);
-    ns = ns < 1 ? 1 : ns;
-    return ns > ns_cap ? ns_cap : ns;
+// Split count for a query tile of the query block: enough splits that each covers about ``chunk`` key tiles.
+__device__ inline int splits_for(int ntiles, int chunk) {
+    const int ns = ceil_div(ntiles, chunk);
+    return ns < 1 ? 1 : ns;
 }
 
 // par: workgroups of the prefill grid per head group, i.e. how many of a plan's items run side by side.
-__global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T, int packed, int par) {
+// pool: split-KV partial slots the caller's workspace has room for (br_split_pool(par)).
+__global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T, int packed, int par, int pool) {
     __shared__ int sh[kPlanThreads / 64];
     __shared__ int s_bad;
     const int tid = threadIdx.x;
@@ -186,13 +182,35 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     }
     int chunk = (int)(w_all / (par > 0 ? par : 1)) - (n_ord > 0 ? (int)(w_ord / n_ord) : 0);
     chunk = chunk < BR_MIN_CHUNK ? BR_MIN_CHUNK : chunk;
+    // ... and long enough that the batch's splits fit the pool of partial slots: lengthen until they do (a chunk
+    // longer than every walk means no split at all, so this ends)
+    for (;;) {
+        int need = 0;
+        for (int b0 = 0; b0 < B; b0 += kPlanThreads) {
+            const int b = b0 + tid;
+            int mine = 0;
+            if (b < B) {
+                const int L = len[b * M + M - 1], pt = M > 1 ? prev_tiles[b] : 0;
+                for (int tt = 0; tt * T < L; ++tt) {
+                    const int e = (tt + 1) * T < L ? (tt + 1) * T : L;
+                    const int ns = splits_for(pt + ceil_div(e, BR_BN), chunk);
+                    mine += ns > 1 ? ns : 0;
+                }
+            }
+            int tot;
+            block_exclusive_scan(mine, sh, &tot);
+            need += tot;
+        }
+        if (need <= pool) break;
+        chunk += (chunk + 1) / 2;
+    }
 
     struct Counts {
-        int glob, x, w, comb;
+        int glob, x, w, comb, slots;
     };
     // what one (sequence, block) pair contributes; pairs are visited sequence by sequence, the query block first
-    auto count_pair = [&](int p, Counts& c, int& b, int& m, int& L, int& nq, int& ns_cap, int& pt, int& npt, bool& is_last) {
-        c = Counts{0, 0, 0, 0};
+    auto count_pair = [&](int p, Counts& c, int& b, int& m, int& L, int& nq, int& pt, int& npt, bool& is_last) {
+        c = Counts{0, 0, 0, 0, 0};
         b = p / M;
         const int jj = p - b * M;
         m = jj == 0 ? M - 1 : jj - 1;
@@ -201,13 +219,12 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         nq = ceil_div(L, T);
         if (is_last) {
             pt = M > 1 ? prev_tiles[b] : 0;
-            ns_cap = nq > 0 ? BR_SLOTS_PER_SEQ / nq : 1;
-            ns_cap = ns_cap < 1 ? 1 : ns_cap;
             for (int tt = 0; tt < nq; ++tt) {
                 int e = (tt + 1) * T < L ? (tt + 1) * T : L;
-                int ns = splits_for(pt + ceil_div(e, BR_BN), ns_cap, chunk);
+                int ns = splits_for(pt + ceil_div(e, BR_BN), chunk);
                 c.glob += ns;
                 c.comb += ns > 1;
+                c.slots += ns > 1 ? ns : 0;
             }
         } else {
             c.x = nq;
@@ -221,11 +238,11 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     long long w_total = 0;
     for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
         const int p = p0 + tid;
-        Counts c = Counts{0, 0, 0, 0};
+        Counts c = Counts{0, 0, 0, 0, 0};
         if (p < BM) {
-            int b, m, L, nq, ns_cap, pt, npt;
+            int b, m, L, nq, pt, npt;
             bool is_last;
-            count_pair(p, c, b, m, L, nq, ns_cap, pt, npt, is_last);
+            count_pair(p, c, b, m, L, nq, pt, npt, is_last);
         }
         int tot;
         block_exclusive_scan(c.glob, sh, &tot);
@@ -240,14 +257,14 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
 
     // Pass 2: the items array is [global queue][XCD queues].
     const int xoff = n_glob_total;
-    int base_glob = 0, base_x = xoff, base_comb = 0;
+    int base_glob = 0, base_x = xoff, base_comb = 0, base_slot = 0;
     long long base_w = 0;
     for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
         const int p = p0 + tid;
-        Counts c = Counts{0, 0, 0, 0};
-        int b = 0, m = 0, L = 0, nq = 0, ns_cap = 1, pt = 0, npt = 0;
+        Counts c = Counts{0, 0, 0, 0, 0};
+        int b = 0, m = 0, L = 0, nq = 0, pt = 0, npt = 0;
         bool is_last = false;
-        if (p < BM) count_pair(p, c, b, m, L, nq, ns_cap, pt, npt, is_last);
+        if (p < BM) count_pair(p, c, b, m, L, nq, pt, npt, is_last);
         int tot;
         int off_g = base_glob + block_exclusive_scan(c.glob, sh, &tot);
         base_glob += tot;
@@ -255,6 +272,8 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         base_x += tot;
         int off_c = base_comb + block_exclusive_scan(c.comb, sh, &tot);
         base_comb += tot;
+        const int off_s = base_slot + block_exclusive_scan(c.slots, sh, &tot);
+        base_slot += tot;
         long long off_w = base_w + block_exclusive_scan(c.w, sh, &tot);
         base_w += tot;
         if (p < BM) {
@@ -269,7 +288,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                 // a block's query tiles are handed out from the last (the longest walk) to the first: what a queue
                 // ends on are short items
                 for (int k = 0; k < nq; ++k) {
-                    const int tt = BR_TILE_ORDER_DESC ? nq - 1 - k : k;
+                    const int tt = nq - 1 - k;
                     it.t0 = tt * T; it.f_lo = 0;
                     it.ntiles = 0x7fffffff; it.slot = -1;
                     items[off_x + k] = it;
@@ -280,12 +299,12 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                 }
             } else {
                 it.nprev = pt;
-                int slot = 0;
+                int slot = off_s;                            // slots of the batch's pool, in item order
                 for (int tt = 0; tt < nq; ++tt) {
                     int e = (tt + 1) * T < L ? (tt + 1) * T : L;
                     int nself = ceil_div(e, BR_BN);
                     int nt = pt + nself;
-                    int ns = splits_for(nt, ns_cap, chunk);
+                    int ns = splits_for(nt, chunk);
                     if (ns > 1) {
                         BrComb cb;
                         cb.b = b; cb.t0 = tt * T; cb.slot0 = slot; cb.nsplit = ns;
@@ -323,6 +342,8 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         hdr[BR_PH_MAX_ITEMS] = max_items;
         hdr[BR_PH_MAX_COMB] = br_plan_max_comb(B);
         hdr[BR_PH_T] = T;
+        hdr[BR_PH_POOL] = pool;
+        hdr[BR_PH_NSLOTS] = base_slot;
     }
 }
 
@@ -340,8 +361,8 @@ __global__ void br_block_table_from_len_kernel(const int* __restrict__ lens, int
 
 }  // namespace
 
-void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int* plan,
-                    hipStream_t stream) {
+void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int pool,
+                    int* plan, hipStream_t stream) {
     int* start = plan + br_plan_off_start();
     int* len = plan + br_plan_off_len(B, M);
     const int BM = B * M;
@@ -353,5 +374,5 @@ void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int 
         hipLaunchKernelGGL(br_block_table_from_len_kernel, dim3((BM + 255) / 256), dim3(256), 0, stream, lens, BM, H,
                            left_padded, start, len);
     }
-    hipLaunchKernelGGL(br_plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, plan, B, M, H, T, packed, par);
+    hipLaunchKernelGGL(br_plan_kernel, dim3(1), dim3(kPlanThreads), 0, stream, plan, B, M, H, T, packed, par, pool);
 }

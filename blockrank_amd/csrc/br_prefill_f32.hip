@@ -119,7 +119,7 @@ __global__ __launch_bounds__(NW * 64) void br_prefill_f32_kernel(BrPrefillParams
 
         if (row_ok) {
             if (it.slot >= 0) {
-                const long long slot = ((long long)b * BR_SLOTS_PER_SEQ + it.slot) * ge.NHG + hg;
+                const long long slot = (long long)it.slot * ge.NHG + hg;
                 const long long prow = slot * (NW * BR_RB) + wave * BR_RB + n;
                 float* po = p.part_o + prow * D + half * HD;
 #pragma unroll
@@ -162,12 +162,12 @@ __global__ __launch_bounds__(256) void br_combine_f32_kernel(BrPrefillParams p, 
             const int head = kvh * ge.G + hsub * ge.Gw + g;
             float mmax = -INFINITY;
             for (int s = 0; s < c.nsplit; ++s) {
-                const long long slot = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0 + s) * ge.NHG + hg;
+                const long long slot = (long long)(c.slot0 + s) * ge.NHG + hg;
                 mmax = fmaxf(mmax, p.part_ml[(slot * rows + r) * 2]);
             }
             float l = 0.f, acc = 0.f;
             for (int s = 0; s < c.nsplit; ++s) {
-                const long long slot = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0 + s) * ge.NHG + hg;
+                const long long slot = (long long)(c.slot0 + s) * ge.NHG + hg;
                 const long long prow = slot * rows + r;
                 const float ms = p.part_ml[prow * 2];
                 const float w8 = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);

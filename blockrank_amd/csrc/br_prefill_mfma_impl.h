@@ -831,7 +831,7 @@ struct Prefill {
         const float lt_tot = lt_run + __shfl_xor(lt_run, 32);    // sum of the rounded probabilities: normalises the output
         if (it.slot >= 0) {
             if (row0 + ln < len_w) {
-                const long long slot = ((long long)b * BR_SLOTS_PER_SEQ + it.slot) * ge.NHG + hg;
+                const long long slot = (long long)it.slot * ge.NHG + hg;
                 const long long prow = slot * (NW * BR_RB) + wave * BR_RB + ln;
                 float* po = p.part_o + prow * D;
 #pragma unroll
@@ -1001,7 +1001,7 @@ __global__ __launch_bounds__(THREADS) void br_finish_kernel(BrPrefillParams p, i
         const int row = c.t0 + sub * BR_RB + rloc;
         if (row >= len_m || hsub * ge.Gw + g >= ge.G) continue;     // (the second: a wave without a head, ragged group)
         const int head = kvh * ge.G + hsub * ge.Gw + g;
-        const long long slot0 = ((long long)c.b * BR_SLOTS_PER_SEQ + c.slot0) * ge.NHG + hg;
+        const long long slot0 = (long long)c.slot0 * ge.NHG + hg;
         const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
         const float2* ml = reinterpret_cast<const float2*>(p.part_ml) + slot0 * rows + r;
         const float* po = p.part_o + (slot0 * rows + r) * D + cc * 4;

@@ -385,7 +385,7 @@ struct PrefillNarrow {
         const float lt_tot = sum_quad(lt_run);              // sum of the rounded probabilities: normalises the output
         if (it.slot >= 0) {
             if (row0 + lr < len_w) {
-                const long long slot = ((long long)b * BR_SLOTS_PER_SEQ + it.slot) * ge.NHG + hg;
+                const long long slot = (long long)it.slot * ge.NHG + hg;
                 const long long prow = slot * (NW / 2 * BR_RB) + ww * BR_RB + half * RW + lr;
                 float* po = p.part_o + prow * D;
 #pragma unroll

@@ -72,7 +72,10 @@ int br_plan_build_from_lengths(const int32_t* lens, int left_padded, int B, int 
 int br_plan_build_packed(const int32_t* lens, int B, int M, int H, int Nq, int Nkv, int32_t* plan, size_t plan_ints,
                          void* stream);
 
-/* Bytes of scratch br_prefill_fwd needs (split-KV partials of the query block). */
+/* Bytes of scratch br_prefill_fwd needs: the split-KV partials of the query blocks' key walks.  The plan cuts those
+ * walks only as far as it takes to give every workgroup of the grid work, and takes the slots from one pool for the
+ * whole batch, so the size follows from the head layout and the current device's compute-unit count and does not grow
+ * with B (about 10 MB for 32 / 8 heads of dim 128 on 256 compute units).  0 without a HIP device. */
 size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D);
 
 /* Block-sparse prefill attention.  Replaces sdpa_blockrank_attention_forward /
@@ -101,12 +104,16 @@ int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out
 /* br_prefill_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
  * result as br_prefill_fwd without the workspace: the split-KV partials live in a device array that
- * belongs to the library (br_prefill_noalloc_max_workspace_bytes() = 80 MiB on every GPU the library is
- * used on, until the process ends).  Neither this call nor anything it calls allocates or frees memory.
- * A request whose br_prefill_workspace_bytes() exceeds that size is refused with BR_ERR_SPACE (Mistral-7B
- * heads: B <= 4).  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
- * streams, two threads) race; calls on one stream, one after the other, do not.  Nothing in the array has
- * to be cleared between calls (a call reads only the partials it wrote itself). */
+ * belongs to the library (br_prefill_noalloc_max_workspace_bytes() = 32 MiB on every GPU the library is
+ * used on, until the process ends).  Neither this call nor anything it calls allocates or frees memory: the
+ * array's address on a device is looked up by the br_plan_build* calls (the first of them on a device loads the
+ * library's code object, which is when the runtime sets the array up), and every request needs a plan, so by the
+ * time this entry runs - under graph capture too - the address is known.
+ * A request whose br_prefill_workspace_bytes() exceeds that size is refused with BR_ERR_SPACE (no head layout
+ * of a current model does: 32 / 8 heads of dim 128 need about 10 MB whatever the batch).  Every call on a GPU
+ * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream,
+ * one after the other, do not.  Nothing in the array has to be cleared between calls (a call reads only the
+ * partials it wrote itself). */
 size_t br_prefill_noalloc_max_workspace_bytes(void);
 int br_prefill_fwd_noalloc(const void* q, const void* k, const void* v, void* out, const int32_t* plan, int B, int Nq,
                            int Nkv, int M, int H, int D, const int64_t* q_strides, const int64_t* k_strides,
