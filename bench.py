@@ -324,6 +324,7 @@ def main():
     ap.add_argument("--backward", action="store_true",
                     help="time the training step of the attention instead: forward that saves the log-sum-exp, then the backward kernels")
     ap.add_argument("--hf-rope", action="store_true", help="cfg3: keep the model file's own rotary embedding (eight elementwise passes per layer)")
+    ap.add_argument("--hinted", action="store_true", help="name the score rows to the hook beforehand (score_rows_hint) instead of letting it guess")
     ap.add_argument("--separate-scores", action="store_true",
                     help="reduce the per-document scores in a launch of their own instead of inside the launch that merges the split partials")
     ap.add_argument("--fused-rope", action="store_true", help="cfg3: rotate Q inside the attention kernel instead of in the stand-alone rotary kernel")
@@ -383,8 +384,20 @@ def main():
         return bench_backward(args, br, layout, wl, q, k, v, mask, scale)
 
     def step(events=None):
-        out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], kernel_events=events,
-                                                      qk_fp8=args.qk_fp8, score_rows_hint=None if args.separate_scores else rows16)
+        # the hook as the reference's callers call it (scripts/eval_attn.py:139: no extra keyword): it guesses the score
+        # rows, the handle confirms the guess against rows16 (once: the tensor is remembered) and returns the scores
+        # the attention call already reduced.  --hinted names the rows beforehand, --separate-scores switches the
+        # guess off (the scores then take a launch of their own).
+        extra = {}
+        if args.separate_scores:
+            extra["speculate_score_rows"] = False
+        elif args.hinted:
+            extra["score_rows_hint"] = rows16
+        if events is not None:
+            extra["kernel_events"] = events
+        if args.qk_fp8:
+            extra["qk_fp8"] = True
+        out, handle = br.blockrank_attention_forward(module, q, k, v, mask, scale, layers_to_return_scores=[20], **extra)
         scores = handle.doc_scores_window(rows16, temperature=0.05) if handle is not None else None
         return out, scores
 

@@ -435,30 +435,109 @@ def doc_scores_from_partials(partials: torch.Tensor, block_mask, rows: torch.Ten
     return (scores, probs) if return_probs else scores
 
 
-class LastBlockScores:
-    """Handle returned in place of the reference's s_last tensor (B, Nq, R, S)
-    (blockrank_std_attention.py:639-645): it keeps the layer's query/key tensors and the block mask so
-    that per-document scores are computed by the fused kernel without writing the logits out.
+_SPEC_ROWS: dict = {}
+# rows tensors found equal to a guess: id -> (weak reference, tensor version, id of the guess).  Kept outside the
+# handles: a serving loop asks every new handle with the same rows tensor, and the comparison costs a host
+# synchronisation.
+_CONFIRMED_ROWS: dict = {}
 
-    ``compute_auxiliary_attention_loss`` of this package accepts it directly; ``dense()`` produces the
-    reference tensor for anything else."""
+
+def _is_confirmed(rows: torch.Tensor, spec: torch.Tensor) -> bool:
+    hit = _CONFIRMED_ROWS.get(id(rows))
+    return hit is not None and hit[0]() is rows and hit[1] == rows._version and hit[2] == id(spec)
+
+
+def _confirm(rows: torch.Tensor, spec: torch.Tensor) -> None:
+    import weakref
+    if len(_CONFIRMED_ROWS) > 256:
+        for key in [k for k, v in _CONFIRMED_ROWS.items() if v[0]() is None]:
+            del _CONFIRMED_ROWS[key]
+    _CONFIRMED_ROWS[id(rows)] = (weakref.ref(rows), rows._version, id(spec))
+
+
+def _speculated_rows(B: int, R: int, device) -> torch.Tensor:
+    """(B, 2) indices {R-2, R-1} into the last R positions of the query block: the rows losses.py:43-48 arrives at
+    whenever the completion is the single "[" token (evaluation: dataset.py:229-249 puts nothing after it), which the
+    attention hook reduces the scores of before anybody has told it the rows.  One tensor per (B, R, device)."""
+    key = (B, R, str(device))
+    t = _SPEC_ROWS.get(key)
+    if t is None:
+        t = torch.tensor([[R - 2, R - 1]] * B, dtype=torch.int32, device=device)
+        _SPEC_ROWS[key] = t
+    return t
+
+
+class LastBlockScores:
+    """What the attention hook returns in place of the reference's s_last tensor (B, Nq, R, S)
+    (blockrank_std_attention.py:639-645).  It keeps the layer's query/key tensors, the block mask and what the
+    attention kernel already left (score partials, and the per-document scores of the rows it was told or guessed),
+    so that ``compute_auxiliary_attention_loss`` of this package gets the scores without the logits ever being
+    written.
+
+    To everything else it behaves as the tensor: shape / dim / size / dtype / device, indexing, any method of
+    torch.Tensor and any torch function (``torch.softmax(h, -1)``, ``h.take_along_dim(...)``, ``h[..., H:-H]``,
+    ``h.float().cpu()``) work on it - the logits are computed when first asked for (``dense()``, fp32) and kept.  The
+    reference's own ``compute_auxiliary_attention_loss`` (losses.py:37-78) therefore runs on it unchanged;
+    ``take_along_dim`` over the row dimension, the first thing that function does, computes just the rows it asks for."""
 
     def __init__(self, query, key, block_mask: BlockMask, scaling: float, num_rows: int, scaled: bool = True, partials=None,
-                 ranked=None):
+                 ranked=None, speculative: bool = False):
         self.query, self.key, self.block_mask = query, key, block_mask
         self.scaling, self.R, self.scaled = float(scaling), int(num_rows), scaled
         self.partials = partials if scaled else None    # per-tile (max, sum) pairs left by the attention kernel
-        # (rows, temperature, scores): per-document scores the attention call already reduced for these rows
+        # (rows, temperature, scores): per-document scores the attention call already reduced for these rows;
+        # speculative: nobody named the rows, they are the hook's guess (_speculated_rows) and have to be compared
         self.ranked = ranked if scaled else None
+        self.speculative = bool(speculative) and self.ranked is not None
+        self._dense = None
         _, Nq, _, D = query.shape
         self.shape = torch.Size((block_mask.B, Nq, self.R, block_mask.M * block_mask.H))
-        self.device, self.dtype = query.device, query.dtype
+        self.device, self.dtype = query.device, torch.float32
 
+    # -- the tensor it stands for -----------------------------------------------------------------
     def dim(self) -> int:
+        return 4
+
+    @property
+    def ndim(self) -> int:
         return 4
 
     def size(self, i=None):
         return self.shape if i is None else self.shape[i]
+
+    def __len__(self):
+        return self.shape[0]
+
+    def __getitem__(self, idx):
+        return self.dense()[idx]
+
+    def __getattr__(self, name):
+        # (reached only for what the handle itself does not define: every other attribute or method of torch.Tensor)
+        if name.startswith("__") or name in ("query", "key", "block_mask", "_dense"):
+            raise AttributeError(name)
+        return getattr(self.dense(), name)
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        def unwrap(x):
+            if isinstance(x, LastBlockScores):
+                return x.dense()
+            if isinstance(x, (list, tuple)):
+                return type(x)(unwrap(y) for y in x)
+            return x
+        return func(*unwrap(args), **{k: unwrap(v) for k, v in (kwargs or {}).items()})
+
+    def take_along_dim(self, indices, dim=None):
+        """Tensor.take_along_dim; the pattern of losses.py:53 - (B, 1, R', 1) row indices over dim 2 - is served by
+        computing those rows' logits alone."""
+        if (dim in (2, -2) and torch.is_tensor(indices) and indices.dim() == 4 and indices.shape[1] == 1 and indices.shape[3] == 1
+                and indices.shape[0] == self.shape[0] and indices.shape[2] <= 16 and self._dense is None and not self.needs_grad()):
+            rows = indices[:, 0, :, 0]
+            # negative indices count from the end, as in torch
+            pos = torch.where(rows < 0, rows + self.R, rows) + (self.block_mask.H - self.R)
+            return last_block_logits(self.query, self.key, self.block_mask, pos.to(torch.int32), self.scaling if self.scaled else 1.0,
+                                     neg=0.7 * torch.finfo(self.query.dtype).min)
+        return self.dense().take_along_dim(indices, dim)
 
     def _rows_default(self) -> torch.Tensor:
         H = self.block_mask.H
@@ -471,28 +550,57 @@ class LastBlockScores:
         """(B, Nq, R, S) logits + additive mask, fp32 unless ``dtype`` is given.  Differentiable with respect
         to the layer's query and key when they require gradients (the auxiliary attention loss of
         trainer.py:79-101 trains through this tensor)."""
-        scale = self.scaling if self.scaled else 1.0
-        neg = 0.7 * torch.finfo(self.dtype).min
-        if self.needs_grad():
-            out = _LastLogitsWithGrad.apply(self.query, self.key, self.block_mask, self._rows_default(), scale, neg)
-        else:
-            out = last_block_logits(self.query, self.key, self.block_mask, self._rows_default(), scale, neg=neg)
+        if self._dense is None:
+            scale = self.scaling if self.scaled else 1.0
+            neg = 0.7 * torch.finfo(self.query.dtype).min
+            if self.needs_grad():
+                self._dense = _LastLogitsWithGrad.apply(self.query, self.key, self.block_mask, self._rows_default(), scale, neg)
+            else:
+                self._dense = last_block_logits(self.query, self.key, self.block_mask, self._rows_default(), scale, neg=neg)
+        out = self._dense
         return out if dtype is None else out.to(dtype)
 
+    # -- the scores -------------------------------------------------------------------------------
     def doc_scores(self, rows: torch.Tensor, temperature: float = 0.05, head_reduce: str = "mean", row_reduce: str = "mean",
                    return_probs: bool = False):
         """Per-document scores for ``rows`` (B, R') positions inside the query block (0..H-1)."""
         return doc_scores(self.query, self.key, self.block_mask, rows, self.scaling if self.scaled else 1.0,
                           temperature=temperature, head_reduce=head_reduce, row_reduce=row_reduce, return_probs=return_probs)
 
+    def speculated_rows(self) -> Optional[torch.Tensor]:
+        """The rows whose scores the attention call reduced on its own guess, or None."""
+        return self.ranked[0] if self.speculative else None
+
+    def confirm_rows(self, rows: torch.Tensor) -> None:
+        """Tell the handle that ``rows`` was compared with ``speculated_rows()`` and found equal (the caller did
+        the comparison together with a check of its own, see losses.compute_auxiliary_attention_loss)."""
+        _confirm(rows, self.ranked[0])
+
+    def _ranked_for(self, rows: torch.Tensor) -> bool:
+        if self.ranked is None:
+            return False
+        if rows is self.ranked[0]:
+            return True
+        if not self.speculative:
+            return False
+        if _is_confirmed(rows, self.ranked[0]):
+            return True
+        # the guess has to be checked against what the caller's labels gave: one small comparison, one host
+        # synchronisation (the reference's own bracket check, losses.py:48, is one too), once per rows tensor
+        spec = self.ranked[0]
+        same = rows.shape == spec.shape and bool((rows.to(device=spec.device, dtype=spec.dtype) == spec).all())
+        if same:
+            _confirm(rows, spec)
+        return same
+
     def doc_scores_window(self, rows: torch.Tensor, temperature: float = 0.05, head_reduce: str = "mean",
                           row_reduce: str = "mean", return_probs: bool = False):
         """Same for ``rows`` (B, R') given as indices 0..R-1 into the handle's own R rows (the last R
-        positions of the query block).  Uses the partials the attention kernel left when there are
-        any (or the scores themselves, when the attention call was told these very rows beforehand); otherwise the
-        stand-alone score kernels."""
-        if (self.ranked is not None and rows is self.ranked[0] and temperature == self.ranked[1] and head_reduce == "mean"
-                and row_reduce == "mean" and not return_probs):
+        positions of the query block).  Uses the scores themselves when the attention call already reduced them for
+        these very rows (it was told them, or guessed them and the guess holds), else the partials the attention
+        kernel left, else the stand-alone score kernels."""
+        if (self.ranked is not None and temperature == self.ranked[1] and head_reduce == "mean" and row_reduce == "mean"
+                and not return_probs and self._ranked_for(rows)):
             return self.ranked[2]
         if self.partials is not None:
             return doc_scores_from_partials(self.partials, self.block_mask, rows, self.R, self.query.shape[1],
@@ -501,6 +609,21 @@ class LastBlockScores:
         pos = (rows + (self.block_mask.H - self.R)).to(torch.int32)
         return self.doc_scores(pos, temperature=temperature, head_reduce=head_reduce, row_reduce=row_reduce,
                                return_probs=return_probs)
+
+
+def _delegate_operator(name):
+    def op(self, *args, **kwargs):
+        return getattr(self.dense(), name)(*args, **kwargs)
+    op.__name__ = name
+    return op
+
+
+# arithmetic and ordering operators are looked up on the type, not through __getattr__: give the handle the tensor's
+# (== and != keep Python's identity semantics, so that a handle stays hashable)
+for _name in ("add", "radd", "sub", "rsub", "mul", "rmul", "truediv", "rtruediv", "pow", "rpow", "matmul", "rmatmul", "neg", "abs",
+              "lt", "le", "gt", "ge", "float", "iter"):
+    setattr(LastBlockScores, f"__{_name}__", _delegate_operator(f"__{_name}__"))
+del _name
 
 
 def _score_args(query, key, block_mask, rows, query_block_only=False):
@@ -667,7 +790,10 @@ def blockrank_attention_forward(
     ``score_rows_hint`` (B, R') int tensor with ``score_temperature`` (default 0.05): the rows (indices into the last
     ``num_last_queries`` positions) the caller is going to ask the handle's ``doc_scores_window`` for with that
     temperature and the default reductions; their scores are then reduced inside the attention call's second launch
-    and the handle returns them when asked with that same tensor object.
+    and the handle returns them when asked with that same tensor object.  Without a hint the hook guesses the last
+    two positions (what losses.py:43-48 yields in evaluation) and the handle checks the guess against the rows it is
+    asked for, falling back to the partials if it was wrong; ``speculate_score_rows=False`` or
+    BLOCKRANK_AMD_NO_SPECULATION=1 switch the guess off.
     """
     assert attention_mask is not None, "BlockRank attention requires an attention mask"
     bm = _as_block_mask(attention_mask)
@@ -715,6 +841,14 @@ def blockrank_attention_forward(
     temperature = float(kwargs.get("score_temperature", 0.05))
     if hint is not None and not 1 <= hint.shape[-1] <= 16:
         hint = None
+    # Nobody named the rows (the reference's callers do not: scripts/eval_attn.py:139): guess the ones losses.py:43-48
+    # yields whenever the completion is the "[" token alone - the last two positions -, reduce their scores in the
+    # attention call's second launch, and let the handle compare the guess with the rows it is later asked for.
+    speculative = False
+    if (hint is None and fuse and bm.M >= 3 and R >= 2 and kwargs.get("speculate_score_rows", True)
+            and not _env_flag("BLOCKRANK_AMD_NO_SPECULATION")):
+        hint = _speculated_rows(bm.B, R, query.device)
+        speculative = True
     out = blockrank_attention(query, key, value, bm, scaling, kernel_events=kwargs.get("kernel_events", None),
                               score_rows=R if fuse else 0, qk_fp8=qk_fp8, q_rope=q_rope, rank_rows=hint,
                               rank_scale=1.0 / (temperature * Nq * hint.shape[-1]) if hint is not None else 1.0)
@@ -726,7 +860,7 @@ def blockrank_attention_forward(
         out, partials = out
     if not want:
         return out, None
-    handle = LastBlockScores(query, key, bm, scaling, R, scaled=scaled, partials=partials, ranked=ranked)
+    handle = LastBlockScores(query, key, bm, scaling, R, scaled=scaled, partials=partials, ranked=ranked, speculative=speculative)
     if needs_grad or kwargs.get("materialize_scores", False) or _env_flag("BLOCKRANK_AMD_DENSE_SCORES"):
         return out, handle.dense()
     return out, handle

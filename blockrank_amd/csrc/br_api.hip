@@ -236,7 +236,7 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     make_geom(Nq, Nkv, &g, &nw, true);
     const size_t rows16 = slots_total(pool, g) * (size_t)nw * BR_RB;
     rows = rows16 > rows ? rows16 : rows;
-    return rows * (size_t)(D + 2) * sizeof(float);
+    return rows * (size_t)(D + 3) * sizeof(float);      // partial outputs, (max, sum) and the exact sum of every row
 }
 
 size_t br_score_partials_bytes(int B, int Nq, int M, int H, int score_rows) {
@@ -339,6 +339,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
     const size_t rows = slots_total(br_split_pool(prefill_par(Nq, Nkv, n_cu)), g) * (size_t)nw * BR_RB;
     p.part_o = static_cast<float*>(workspace);
     p.part_ml = p.part_o + rows * D;
+    p.part_lx = p.part_ml + rows * 2;
     p.sq_b = q_strides[0]; p.sq_h = q_strides[1]; p.sq_t = q_strides[2];
     p.sk_b = k_strides[0]; p.sk_h = k_strides[1]; p.sk_t = k_strides[2];
     p.sv_b = v_strides[0]; p.sv_h = v_strides[1]; p.sv_t = v_strides[2];

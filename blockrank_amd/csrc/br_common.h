@@ -247,7 +247,10 @@ struct BrPrefillParams {
     void* out;
     const int* plan;
     float* part_o;    // split-KV partial outputs: [slot][NW*32 rows][D] fp32, unnormalised
-    float* part_ml;   // [slot][NW*32 rows][2]: running max (log2 domain) and denominator
+    float* part_ml;   // [slot][NW*32 rows][2]: running max (log2 domain) and denominator (the sum of the probabilities as
+                      // rounded for the P V product: what normalises the merged output)
+    float* part_lx;   // [slot][NW*32 rows]: the exact sum of the probabilities, written and read only when the
+                      // log-sum-exp is asked for (lse below)
     long long sq_b, sq_h, sq_t;   // element strides of q for (batch, head, token); the last dim is dense
     long long sk_b, sk_h, sk_t;
     long long sv_b, sv_h, sv_t;

@@ -844,6 +844,7 @@ struct Prefill {
                 if (lh == 0) {
                     p.part_ml[prow * 2] = m_run;
                     p.part_ml[prow * 2 + 1] = lt_tot;
+                    if (SC && p.lse != nullptr) p.part_lx[prow] = l_tot;
                 }
             }
         } else {
@@ -1004,36 +1005,42 @@ __global__ __launch_bounds__(THREADS) void br_finish_kernel(BrPrefillParams p, i
         const long long slot0 = (long long)c.slot0 * ge.NHG + hg;
         const long long sstride = (long long)ge.NHG * rows;          // rows between consecutive splits
         const float2* ml = reinterpret_cast<const float2*>(p.part_ml) + slot0 * rows + r;
+        const float* lx = p.part_lx + slot0 * rows + r;
+        const bool want_lse = p.lse != nullptr && cc == 0;
         const float* po = p.part_o + (slot0 * rows + r) * D + cc * 4;
         // all loads of up to eight splits are in flight together; a thread owns one float4 of the row
-        float mmax = -INFINITY, l = 0.f;
+        float mmax = -INFINITY, l = 0.f, lex = 0.f;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         for (int s0 = 0; s0 < c.nsplit; s0 += 8) {
             float2 mls[8];
+            float lxs[8];
             f32x4 ov[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const bool on = s0 + j < c.nsplit;
                 mls[j] = on ? ml[(s0 + j) * sstride] : make_float2(-INFINITY, 0.f);
                 ov[j] = on ? *reinterpret_cast<const f32x4*>(po + (s0 + j) * sstride * D) : f32x4{0.f, 0.f, 0.f, 0.f};
+                lxs[j] = (on && want_lse) ? lx[(s0 + j) * sstride] : 0.f;
             }
             float mnew = mmax;
 #pragma unroll
             for (int j = 0; j < 8; ++j) mnew = fmaxf(mnew, mls[j].x);
             const float resc = mmax == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mmax - mnew);
             l *= resc;
+            lex *= resc;
             acc *= resc;
             mmax = mnew;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float w8 = mls[j].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mls[j].x - mmax);
                 l += mls[j].y * w8;
+                lex += lxs[j] * w8;
                 acc += ov[j] * w8;
             }
         }
         const float inv = l > 0.f ? 1.f / l : 0.f;
-        if (p.lse != nullptr && cc == 0)
-            p.lse[(long long)c.b * p.lse_b + (long long)head * p.lse_h + qtok0 + row] = mmax + __builtin_amdgcn_logf(l);
+        // (the log-sum-exp from the exact sums, as the rows the prefill kernel finishes itself get it)
+        if (want_lse) p.lse[(long long)c.b * p.lse_b + (long long)head * p.lse_h + qtok0 + row] = mmax + __builtin_amdgcn_logf(lex);
         BR_E16* dst = reinterpret_cast<BR_E16*>(p.out) + (long long)c.b * p.so_b + (long long)head * p.so_h +
                       (long long)(qtok0 + row) * p.so_t;
         e16x4 h4 = __builtin_convertvector(acc * inv, e16x4);

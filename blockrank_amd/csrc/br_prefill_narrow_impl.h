@@ -390,6 +390,12 @@ struct PrefillNarrow {
                 float* po = p.part_o + prow * D;
 #pragma unroll
                 for (int d = 0; d < D / 16; ++d) *reinterpret_cast<f32x4*>(po + d * 16 + 4 * lg) = o[d];
+                if constexpr (SC) {
+                    if (lse_out) {
+                        const float l_tot = sum_quad(l_run);
+                        if (lg == 0) p.part_lx[prow] = l_tot;
+                    }
+                }
                 if (lg == 0) {
                     p.part_ml[prow * 2] = m_run;
                     p.part_ml[prow * 2 + 1] = lt_tot;

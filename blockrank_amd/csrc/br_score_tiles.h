@@ -108,8 +108,10 @@ __device__ __forceinline__ void br_doc_final_tiles_body(const BrTileScoreParams&
 #pragma unroll
         for (int k = 0; k < DPL; ++k) {
             const int d = lane + 64 * k;
-            t0m[k] = d < docs ? tbase[b * p.M + d + 1] : 0;
             ntm[k] = d < docs ? (len[b * p.M + d + 1] + BR_BN - 1) / BR_BN : 0;
+            // (a document without tokens owns no tile: its loads below go to the row's first partial, not to the index
+            // one past the documents before it, which for trailing empty documents is one past the row's partials)
+            t0m[k] = ntm[k] > 0 ? tbase[b * p.M + d + 1] : 0;
         }
         for (int j0 = wave; j0 < NR; j0 += PG * nwaves) {
             float md[PG][DPL], sdm[PG][DPL];

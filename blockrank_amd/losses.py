@@ -14,14 +14,20 @@ import torch.nn.functional as F
 from .attention import LastBlockScores
 
 
-def bracket_rows(labels: torch.Tensor, h1: int) -> torch.Tensor:
+def bracket_rows(labels: torch.Tensor, h1: int, guess: torch.Tensor | None = None, return_match: bool = False):
     """(B, S) labels -> (B, 2) indices into the last h1 positions: the first label > -100 (the "["
-    token) and the position before it (losses.py:43-48)."""
+    token) and the position before it (losses.py:43-48).  With ``guess`` (B, 2) and ``return_match`` also whether the
+    rows equal it, found out in the same host synchronisation as the reference's bracket check."""
     last = labels[:, -h1:] > -100
     br = last.int().argmax(dim=-1)[:, None]
     rows = torch.hstack([br - 1, br])
-    assert torch.all(rows >= 0), "Bracket token not found in last h1 positions."
-    return rows
+    if guess is None or not return_match:
+        assert torch.all(rows >= 0), "Bracket token not found in last h1 positions."
+        return (rows, False) if return_match else rows
+    same = (rows == guess.to(rows.device)).all() if rows.shape == guess.shape else torch.zeros((), dtype=torch.bool, device=rows.device)
+    ok, match = torch.stack([torch.all(rows >= 0), same]).tolist()
+    assert ok, "Bracket token not found in last h1 positions."
+    return rows, bool(match)
 
 
 def _infonce(logits: torch.Tensor, answer_ids: torch.Tensor, return_logits: bool):
@@ -59,7 +65,10 @@ def compute_auxiliary_attention_loss(
     _, N, h1, MH = attention_scores.shape
     assert MH == M * H, "Attention scores last dimension must match M*H"
     if rows is None:
-        rows = bracket_rows(labels, h1)                              # (B, 2) in [0, h1)
+        guess = attention_scores.speculated_rows() if isinstance(attention_scores, LastBlockScores) else None
+        rows, match = bracket_rows(labels, h1, guess, return_match=True)     # (B, 2) in [0, h1)
+        if match:
+            attention_scores.confirm_rows(rows)              # the attention call's own guess holds: its scores are these rows'
     if isinstance(attention_scores, LastBlockScores) and attention_scores.needs_grad():
         attention_scores = attention_scores.dense()          # training: the differentiable logits tensor
     if isinstance(attention_scores, LastBlockScores):

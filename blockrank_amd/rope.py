@@ -129,8 +129,17 @@ def patch_rotary(model, fuse_q: bool = False) -> list[str]:
     """Replace ``apply_rotary_pos_emb`` in the module(s) that define the attention classes of ``model`` (a
     Hugging Face decoder).  Returns the names of the patched modules; ``unpatch_rotary`` restores them.
     ``fuse_q=True`` installs ``apply_rotary_pos_emb_fused`` instead: K is rotated by the kernel here, Q by the
-    attention kernel (the model's attention implementation must be one of this package's BlockRank names)."""
+    attention kernel: the model's attention implementation must be one of this package's BlockRank names (checked here;
+    call ``unpatch_rotary`` before switching the model to another implementation)."""
     fn = apply_rotary_pos_emb_fused if fuse_q else apply_rotary_pos_emb
+    if fuse_q:
+        # the unrotated Q the fused function returns is only completed by this package's attention hook: under any
+        # other attention implementation it would be consumed as it is, silently wrong
+        from .attention import STD_IMPL_NAMES, TRITON_IMPL_NAMES
+        impl = getattr(getattr(model, "config", None), "_attn_implementation", None)
+        if impl not in STD_IMPL_NAMES + TRITON_IMPL_NAMES:
+            raise ValueError(f"patch_rotary(fuse_q=True) needs one of the BlockRank attention implementations, the model uses {impl!r}; "
+                             "set it first (and call unpatch_rotary before switching to another one)")
     done = []
     for m in model.modules():
         mod = sys.modules.get(type(m).__module__)

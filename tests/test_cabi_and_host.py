@@ -151,3 +151,33 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_scores_handle_is_a_tensor_to_strangers(monkeypatch):
+    """LastBlockScores in place of the reference's s_last tensor: torch functions, methods and indexing reach the
+    logits (here a stub of the logits kernel, so that the protocol itself is checked without a GPU)."""
+    import types
+    from blockrank_amd import attention as att
+    B, Nq, R, M, H, D = 2, 4, 16, 5, 32, 64
+    g = torch.Generator().manual_seed(0)
+    full = torch.randn(B, Nq, H, M * H, generator=g)                       # logits of every query-block position
+
+    def fake_logits(query, key, bm, rows, scaling, neg=None):
+        return full.take_along_dim(rows.long()[:, None, :, None], dim=2)
+
+    monkeypatch.setattr(att, "last_block_logits", fake_logits)
+    bm = types.SimpleNamespace(B=B, M=M, H=H)
+    h = att.LastBlockScores(torch.zeros(B, Nq, M * H, D), torch.zeros(B, 2, M * H, D), bm, 0.125, R)
+    want = full[:, :, H - R:]
+    idx = torch.tensor([[14, 15], [3, 4]])[:, None, :, None]
+    got = h.take_along_dim(idx, dim=2)
+    assert h._dense is None and torch.equal(got, want.take_along_dim(idx, dim=2))
+    assert torch.equal(h.take_along_dim(torch.tensor([[-1, -2], [0, 1]])[:, None, :, None], dim=2),
+                       want.take_along_dim(torch.tensor([[15, 14], [0, 1]])[:, None, :, None], dim=2))
+    assert tuple(h.shape) == (B, Nq, R, M * H) and h.dim() == 4 and h.size(-1) == M * H and len(h) == B
+    assert torch.equal(h[..., H:-H], want[..., H:-H])
+    assert torch.equal(torch.softmax(h, dim=-1), torch.softmax(want, dim=-1))
+    assert torch.equal(torch.nn.functional.softmax(h[..., H:-H], dim=-1), torch.softmax(want[..., H:-H], dim=-1))
+    assert torch.equal(h * 2, want * 2) and torch.equal(h.double(), want.double()) and torch.allclose(h.mean(dim=(1, 2)), want.mean(dim=(1, 2)), atol=1e-6)
+    with pytest.raises(AttributeError):
+        h.no_such_attribute

@@ -70,6 +70,28 @@ def test_saved_log_sum_exp_matches_oracle():
     assert np.abs(lse[rows] - want[rows]).max() <= 2e-3
 
 
+def test_log_sum_exp_of_split_rows_is_exact_too():
+    # one request with many documents: the query block's key walk is cut into several items and its rows' log-sum-exp
+    # comes from the merge of their partials.  Peaked rows (large logits: one key carries the mass, so the sum of the
+    # bf16-rounded probabilities that normalises the output is off from the exact one by up to 2^-9) must come out as
+    # exact as the rows a single item finishes: 1e-4 in natural-log units.
+    lay = synthetic.random_layout(1, 48, 40, 30, 96, 24, seed=8)
+    Nq, Nkv, D = 8, 2, 128
+    q, k, v = synthetic.random_qkv(lay, Nq, Nkv, D, torch.bfloat16, DEV, seed=5)
+    q = (q * 6).contiguous()
+    qq = q.clone().requires_grad_(True)
+    out = br.blockrank_attention(qq, k, v, br.BlockMask(lay.valid.to(DEV), torch.bfloat16), D ** -0.5)
+    lse = out.grad_fn.saved_tensors[4].cpu().double().numpy() * math.log(2.0)
+    *_, want = orc.dense_attention_backward(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(),
+                                            np.zeros((lay.B, lay.S, Nq, D)), lay.valid.numpy(), D ** -0.5)
+    rows = np.broadcast_to(real_rows(lay).numpy()[:, None, :], want.shape)
+    err = np.abs(lse - want)
+    assert err[rows].max() <= 1e-4
+    last = np.zeros_like(rows)
+    last[:, :, -lay.H:] = rows[:, :, -lay.H:]                    # the query block's rows: the split ones
+    assert last.any() and err[last].max() <= 1e-4
+
+
 def test_ragged_blocks_four_heads_per_group():
     _check(synthetic.make_layout([[40, 100, 160, 33, 192, 20], [64, 7, 150, 90, 0, 31]]), 8, 2, 128)
 
