@@ -65,6 +65,9 @@ def workloads():
         # the headline layout with eight query heads per kv head (Llama-3-70B-like grouping)
         "cfg2g8": dict(desc="cfg2 layout with 32q/4kv heads (8 per group), D=128, bf16", layout=lambda: synthetic.uniform_layout(4, 64, 20, 160, 32),
                        Nq=32, Nkv=4, D=128, hidden=None, dtype=torch.bfloat16),
+        # the ragged layout of the end-to-end request (BASELINE config 3), one attention layer of it
+        "cfg3layout": dict(desc="Mistral-7B attention shapes, B=8, 64-token prefix + 20 docs U[96,224] + 32-token query, bf16 (the end-to-end request's layout)",
+                           layout=lambda: synthetic.random_layout(8, 64, 20, 96, 224, 32, seed=0), Nq=32, Nkv=8, D=128, hidden=None, dtype=torch.bfloat16),
         # the small fp32 case that also runs on a CPU in seconds
         "cfg1": dict(desc="fp32, B=1, 8q/2kv heads, D=64, 32-token prefix + 8 docs x 64 + 16-token query", layout=lambda: synthetic.uniform_layout(1, 32, 8, 64, 16),
                      Nq=8, Nkv=2, D=64, hidden=None, dtype=torch.float32),
@@ -177,6 +180,7 @@ def run_model(args, steps, warmup):
     if not args.hf_layer_ops:
         br.patch_layer_ops(model)        # one-pass RMSNorm and SiLU-gate kernels instead of the model file's eager expressions
         br.patch_qkv(model)              # one GEMM for the Q, K and V projections of a layer
+    extra = {}
     if args.padded:
         def forward(**kw):
             return ranker(ids, valid, pos, rows=rows, **kw)
@@ -208,6 +212,72 @@ def run_model(args, steps, warmup):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     assert torch.isfinite(scores).all()
+
+    def timed_each(fn, n):
+        """Median of n calls, each waited for: what one caller sees from call to result."""
+        ts = []
+        for _ in range(n):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t1) * 1e3)
+        ts.sort()
+        return ts[len(ts) // 2]
+
+    def graph_of(fn):
+        """The forward captured in a HIP graph (everything the host would have to look at is prepared beforehand);
+        returns (replay, result) or None where the capture does not go through."""
+        try:
+            g = torch.cuda.CUDAGraph()
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                fn()
+                torch.cuda.synchronize()
+                with torch.cuda.graph(g, stream=s):
+                    out = fn()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            return g.replay, out
+        except Exception as e:          # a library call inside the model that cannot be captured: report, do not fail the run
+            sys.stderr.write(f"HIP graph capture of the forward failed: {e}\n")
+            torch.cuda.synchronize()
+            return None
+
+    # Ranking latency: one request (the first sequence of the batch) through the same layers, call to result; and the
+    # share of the eager forward's wall time that replaying the very same kernels from a HIP graph does not need (the
+    # GPU idling between eager launches).
+    if not args.padded:
+        prep = ranker.prepare_packed(lens_dev, layout.H)
+        lay1 = synthetic.make_layout([list(layout.lengths[0])], H=layout.H)
+        keep1 = lay1.valid.reshape(-1)
+        ids1 = ids[:1].reshape(-1)[keep1.to(dev)][None]
+        pos1 = lay1.position_ids.reshape(-1)[keep1][None].to(dev)
+        lens1 = torch.as_tensor(lay1.lengths, dtype=torch.int32, device=dev)
+        prep1 = ranker.prepare_packed(lens1, layout.H)
+        rows1 = rows[:1].contiguous()
+
+        def forward1(**kw):
+            return ranker.forward_packed(ids1, pos1, lens1, rows1, H=layout.H, prepared=prep1, **kw)
+
+        for _ in range(3):
+            forward1()
+        extra["latency_ms_b1"] = timed_each(forward1, 15)
+        extra["ms_per_batch_each"] = timed_each(lambda: forward(prepared=prep), 5)
+        g8 = graph_of(lambda: forward(prepared=prep))
+        if g8 is not None:
+            replay8, out8 = g8
+            assert torch.allclose(out8, scores, rtol=1e-3, atol=1e-5), "graph replay changed the scores"
+            extra["ms_per_batch_graph"] = timed_each(replay8, 5)
+            extra["gpu_idle_frac"] = max(0.0, 1.0 - extra["ms_per_batch_graph"] / extra["ms_per_batch_each"])
+            del g8, replay8, out8
+        g1 = graph_of(forward1)
+        if g1 is not None:
+            extra["latency_ms_b1_graph"] = timed_each(g1[0], 15)
+            extra["gpu_idle_frac_b1"] = max(0.0, 1.0 - extra["latency_ms_b1_graph"] / extra["latency_ms_b1"])
+            del g1
     # the attention kernel of every layer of one more forward, from HIP events around it
     pairs = []
 
@@ -252,6 +322,7 @@ def run_model(args, steps, warmup):
         "roofline_hbm": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "bytes_per_launch": alg_bytes},
     }
+    res.update(extra)
     return res
 
 
@@ -332,6 +403,13 @@ def main():
                     help="cfg3: keep the model file's own RMSNorm and SiLU-gate expressions (ten elementwise passes per layer)")
     ap.add_argument("--padded", action="store_true",
                     help="cfg3: feed the reference's padded (B, M, H) batch instead of the packed one")
+    ap.add_argument("--packed-layout", action="store_true",
+                    help="single-layer workloads: feed the packed token layout (real tokens only) instead of the padded (B, M, H) one")
+    ap.add_argument("--alias-kv", action="store_true",
+                    help="measurement aid (results are wrong): K and V with a token stride of 0, so that every key row is the same 256 cached "
+                         "bytes - what is left of the kernel's HBM traffic is the Q and output streams")
+    ap.add_argument("--alias-q", action="store_true", help="measurement aid (results are wrong): Q with a token stride of 0 - what is left of the "
+                                                           "HBM reads is the K/V stream")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times, so that a profiler's HBM byte counters can be "
                          "scaled against a kernel of known traffic")
@@ -363,11 +441,22 @@ def main():
     R = min(16, layout.H)
     rows16 = torch.tensor([[R - 2, R - 1]] * layout.B, dtype=torch.int32, device=dev)   # "[" and the token before it, in the last 16 positions
     module = _Module(20, Nq // Nkv)
+    if args.packed_layout:
+        # real tokens only, all blocks of all sequences one after the other on one token axis: (1, heads, T, D)
+        q, k, v = (t.transpose(1, 2)[valid.reshape(layout.B, layout.S)][None].transpose(1, 2) for t in (q, k, v))
+        lens_dev = torch.as_tensor(layout.lengths, dtype=torch.int32, device=dev)
+    if args.alias_kv:
+        k, v = k[:, :, :1].expand_as(k), v[:, :, :1].expand_as(v)
+    if args.alias_q:
+        q = q[:, :, :1].expand_as(q)
 
     # once per forward pass: mask hook -> plan
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    mask = br.blockrank_attention_mask(batch_size=layout.B, attention_mask=valid, dtype=dtype)
+    if args.packed_layout:
+        mask = br.BlockMask.from_lengths(lens_dev, H=layout.H, packed=True, dtype=dtype)
+    else:
+        mask = br.blockrank_attention_mask(batch_size=layout.B, attention_mask=valid, dtype=dtype)
     mask.plan(Nq, Nkv)
     torch.cuda.synchronize()
     plan_ms = (time.perf_counter() - t0) * 1e3
@@ -470,7 +559,11 @@ def main():
         "dtype": ("fp8 e4m3 (Q K^T) + bf16 (P V)" if args.qk_fp8 else "bf16") if dtype == torch.bfloat16 else "f32",
         "data": "synthetic",
         "config": {"workload": wl["desc"], "name": args.workload, "batch": layout.B, "blocks": layout.M, "block_len": layout.H,
-                   "valid_tokens": layout.valid_tokens, "unmasked_pairs": pairs_n, "launch": "graph" if graph_ms is not None and graph_ms < ms_per_step else "eager"},
+                   "valid_tokens": layout.valid_tokens, "unmasked_pairs": pairs_n, "launch": "graph" if graph_ms is not None and graph_ms < ms_per_step else "eager",
+                   "token_layout": "packed (real tokens only)" if args.packed_layout else "padded (B, M, H)",
+                   "score_rows": "named beforehand (score_rows_hint)" if args.hinted else ("reduced in a launch of their own" if args.separate_scores
+                                                                                       else "guessed by the hook, confirmed by the handle"),
+                   **({"aliased": "K/V" if args.alias_kv else "Q"} if (args.alias_kv or args.alias_q) else {})},
         "prefill_tok_per_s": layout.valid_tokens / (best_ms * 1e-3),
         "ms_per_step_eager": ms_per_step,
         "ms_per_step_graph": graph_ms,
@@ -484,9 +577,16 @@ def main():
     }
     if dtype == torch.float32:
         res["roofline"].update(bound="mfma", peak=157.3, frac=tflops / 157.3, kernel="br_prefill_f32_kernel")
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not (args.packed_layout or args.alias_kv or args.alias_q):
         res["cpu_baseline"] = cpu_baseline(layout, q, k, v, scale, dtype)
         res["cpu_baseline"]["gpu_over_cpu"] = res["value"] / res["cpu_baseline"]["value"]
+        if args.workload == "cfg2" and dtype == torch.bfloat16:
+            # the same request in fp32 (the dtype the reference's CPU path is quoted in) and BASELINE config 1, both bounded
+            res["cpu_baseline"]["fp32"] = cpu_baseline(layout, q, k, v, scale, torch.float32, budget_s=5.0)
+            w1 = workloads()["cfg1"]
+            lay1 = w1["layout"]()
+            q1, k1, v1 = synthetic.random_qkv(lay1, w1["Nq"], w1["Nkv"], w1["D"], torch.float32, dev)
+            res["cpu_baseline"]["cfg1_fp32"] = cpu_baseline(lay1, q1, k1, v1, w1["D"] ** -0.5, torch.float32, budget_s=2.0)
     if args.workload == "cfg2" and not args.no_e2e and not args.qk_fp8:
         # the ranking request end to end: what the headline layer is one twenty-first of
         del q, k, v, out, scores
@@ -501,6 +601,9 @@ def main():
             "attention_roofline_frac_mfma": m["roofline"]["frac"], "attention_roofline_frac_hbm": m["roofline_hbm"]["frac"],
             "dense_tflops": m["dense_tflops"],
         }
+        for key in ("latency_ms_b1", "latency_ms_b1_graph", "ms_per_batch_each", "ms_per_batch_graph", "gpu_idle_frac", "gpu_idle_frac_b1"):
+            if key in m:
+                res["e2e"][key] = m[key]
     print(json.dumps(res))
 
 

@@ -107,13 +107,29 @@ class TruncatedRanker:
         q, _ = rope(q, q, cos[:, S - H:], sin[:, S - H:])
         return doc_scores(q, k, mask, pos, attn.scaling, temperature=self.temperature, query_block_only=True)
 
+    def prepare_packed(self, block_lengths: torch.Tensor, H: Optional[int] = None, dtype: torch.dtype = torch.bfloat16) -> dict:
+        """Everything about a packed batch that depends on the block lengths alone and needs the host to look at
+        them: the block mask with its device plan and the positions of the query blocks' tokens on the token axis.
+        ``forward_packed(..., prepared=...)`` then runs without a host synchronisation, so it can be captured in a
+        HIP graph and replayed for every batch of that shape."""
+        B, M = block_lengths.shape
+        dev = block_lengths.device
+        mask = BlockMask.from_lengths(block_lengths, H=H, packed=True, dtype=dtype)
+        cfg = self.base.config
+        mask.plan(cfg.num_attention_heads, cfg.num_key_value_heads)
+        flat = block_lengths.reshape(-1).long()
+        block_of = torch.repeat_interleave(torch.arange(B * M, device=dev), flat, output_size=mask.total_tokens)
+        idx_q = ((block_of % M) == M - 1).nonzero().squeeze(-1)
+        return dict(mask=mask, idx_q=idx_q)
+
     @torch.no_grad()
     def forward_packed(self, input_ids: torch.Tensor, position_ids: torch.Tensor, block_lengths: torch.Tensor, rows: torch.Tensor,
-                       H: Optional[int] = None, **layer_kwargs) -> torch.Tensor:
+                       H: Optional[int] = None, prepared: Optional[dict] = None, **layer_kwargs) -> torch.Tensor:
         """The same forward on a packed batch (see blockrank_amd.collate): input_ids, position_ids (1, T)
         hold the real tokens only, block_lengths (B, M) says how they split into blocks, rows (B, R)
         are indices into the last ``num_last_queries`` positions of the query block.  The dense layers
-        then run over T tokens instead of B*M*H slots.  Returns (B, M-2) fp32 scores."""
+        then run over T tokens instead of B*M*H slots.  ``prepared``: the result of ``prepare_packed`` for these
+        block lengths (the call then never waits for the device).  Returns (B, M-2) fp32 scores."""
         base = self.base
         B, M = block_lengths.shape
         assert M >= 3, "ranking needs a prefix, at least one document and a query block"
@@ -122,7 +138,9 @@ class TruncatedRanker:
         input_ids = input_ids.reshape(1, T)
         position_ids = position_ids.reshape(1, T)
         hidden = base.embed_tokens(input_ids)
-        mask = BlockMask.from_lengths(block_lengths.to(dev), H=H, packed=True, dtype=hidden.dtype)
+        if prepared is None:
+            prepared = self.prepare_packed(block_lengths.to(dev), H, hidden.dtype)
+        mask = prepared["mask"]
         assert mask.total_tokens == T, "block_lengths do not sum to the number of tokens"
         Hs = mask.H
         h1 = self.num_last_queries if Hs >= self.num_last_queries else Hs
@@ -146,9 +164,7 @@ class TruncatedRanker:
         _, k = rope(k, k, cos, sin)
         # queries of the query blocks only, scattered to their places on the token axis (the score
         # kernels read no other query rows, so the rest of that buffer stays unwritten)
-        flat = block_lengths.to(dev).reshape(-1).long()
-        block_of = torch.repeat_interleave(torch.arange(B * M, device=dev), flat, output_size=T)
-        idx_q = ((block_of % M) == M - 1).nonzero().squeeze(-1)
+        idx_q = prepared["idx_q"]
         qc = attn.q_proj(x[:, idx_q]).view(1, idx_q.numel(), -1, D).transpose(1, 2)
         qc, _ = rope(qc, qc, cos[:, idx_q], sin[:, idx_q])
         Nq = qc.shape[1]
