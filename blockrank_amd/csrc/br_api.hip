@@ -12,9 +12,9 @@
 void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int pool,
                     int* plan, hipStream_t stream);
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank, int wave_rows);
+                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
 int br_launch_prefill_f16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                          hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank, int wave_rows);
+                          hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank);
 int br_launch_prefill_f32(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
                            hipEvent_t ev_start, hipEvent_t ev_stop);
 int br_launch_doc_scores(const void* q, const void* k, const int* plan, const int* rows, float* part, float* scores,
@@ -130,12 +130,20 @@ int check_strides(const char* name, const int64_t* s, int dtype) {
 
 // Workgroups of the 16-bit prefill grid that share one head group's items: what the plan balances the split of the
 // query blocks' walks against, and what sizes the pool of split-KV partial slots.
-int prefill_par(int Nq, int Nkv, int n_cu) {
+int prefill_par(int Nq, int Nkv, int n_cu, int* nhg = nullptr) {
     BrGeom g16;
     int nw16;
     if (!make_geom(Nq, Nkv, &g16, &nw16, true)) return 1;
+    if (nhg) *nhg = g16.NHG;
     const int par = n_cu * prefill_wgs_per_cu(nw16) / g16.NHG;
     return par < 1 ? 1 : par;
+}
+
+// Slots of the split-KV partial pool for a head layout on the current device.
+int prefill_pool(int Nq, int Nkv, int n_cu) {
+    int nhg = 1;
+    const int par = prefill_par(Nq, Nkv, n_cu, &nhg);
+    return br_split_pool(par, nhg);
 }
 
 size_t slots_total(int pool, const BrGeom& g) { return (size_t)pool * g.NHG; }
@@ -194,7 +202,7 @@ static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded
     BrGeom g16;
     int nw16;
     make_geom(Nq, Nkv, &g16, &nw16, true);                  // the shape the 16-bit forward kernels run in
-    if ((long long)br_plan_max_items(B, M, H, T) * (g16.NHG > g.NHG ? g16.NHG : g.NHG) >= (1 << 24))
+    if ((long long)br_plan_max_items(B, M, H, T) * (g16.NHG > g.NHG ? g16.NHG : g.NHG) >= (1 << 24) || B > 1024)
         return fail(BR_ERR_ARG, "batch too large for one plan (B=%d, M=%d, H=%d)", B, M, H);
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");
@@ -204,7 +212,7 @@ static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded
     int src = noalloc_scratch(&scratch_ptr);
     if (src) return src;
     const int par = prefill_par(Nq, Nkv, n_cu);
-    br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, par, br_split_pool(par), plan, static_cast<hipStream_t>(stream));
+    br_launch_plan(valid, lens, left_padded, packed, B, M, H, T, par, prefill_pool(Nq, Nkv, n_cu), plan, static_cast<hipStream_t>(stream));
     return check_launch("plan launch");
 }
 
@@ -230,7 +238,7 @@ size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D) {
     if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || D <= 0) return 0;
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return 0;
-    const int pool = br_split_pool(prefill_par(Nq, Nkv, n_cu));
+    const int pool = prefill_pool(Nq, Nkv, n_cu);
     size_t rows = slots_total(pool, g) * (size_t)nw * BR_RB;
     // (the 16-bit kernels may cut a head group differently from the fp32 kernel: enough for either)
     make_geom(Nq, Nkv, &g, &nw, true);
@@ -336,7 +344,7 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
 
     BrPrefillParams p;
     p.q = q; p.k = k; p.v = v; p.out = out; p.plan = plan;
-    const size_t rows = slots_total(br_split_pool(prefill_par(Nq, Nkv, n_cu)), g) * (size_t)nw * BR_RB;
+    const size_t rows = slots_total(prefill_pool(Nq, Nkv, n_cu), g) * (size_t)nw * BR_RB;
     p.part_o = static_cast<float*>(workspace);
     p.part_ml = p.part_o + rows * D;
     p.part_lx = p.part_ml + rows * 2;
@@ -398,10 +406,8 @@ static int prefill_impl(const void* q, const void* k, const void* v, void* out, 
         p.qk_scales = scales;
         lrc = br_launch_prefill_fp8qk(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp);
     } else {
-        const char* wr_env = getenv("BLOCKRANK_AMD_WAVE_ROWS");
-        const int wave_rows = wr_env ? atoi(wr_env) : 32;
-        lrc = dtype == BR_DTYPE_BF16  ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp, wave_rows)
-              : dtype == BR_DTYPE_F16 ? br_launch_prefill_f16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp, wave_rows)
+        lrc = dtype == BR_DTYPE_BF16  ? br_launch_prefill_bf16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
+              : dtype == BR_DTYPE_F16 ? br_launch_prefill_f16(p, D, nw, n_cu, combine_grid, s, e0, e1, rankp)
                                       : br_launch_prefill_f32(p, D, nw, n_cu, combine_grid, s, e0, e1);
     }
     if (lrc) return fail(BR_ERR_ARG, "no kernel for head dim %d with %d query heads per kv head", D, g.G);

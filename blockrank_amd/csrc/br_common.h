@@ -14,7 +14,7 @@
 #define BR_RB 32              // query rows per wave (one 32x32 MFMA row block)
 // Split-KV partial slots of the query blocks' key walks: one pool for the whole batch, handed out by the plan in
 // item order.  Splitting exists to give every workgroup of the grid something to do, so the pool is a fraction of
-// the workgroups that share a head group's items (par) and does not grow with the batch: br_split_pool(par) slots,
+// the workgroups that share a head group's items (par) and does not grow with the batch: br_split_pool(par, nhg) slots,
 // at most BR_SPLIT_POOL_MAX.  The plan lengthens the splits until the batch fits the pool.
 #define BR_SPLIT_POOL_MAX 160
 #ifndef BR_MIN_CHUNK
@@ -22,16 +22,17 @@
 #endif
 
 // Plan buffer (int32):
-//   [header BR_PLAN_HDR][start B*M][len B*M][tok B*M][prev_tiles B][tile base B*M][tile descriptors 2*B*TPS]
-//   [items 16*max_items][comb 4*max_comb]
-// The items array holds the query-block items (global queue) followed by the items of all other blocks
-// (XCD queues).
+//   [header BR_PLAN_HDR][start B*M][len B*M][tok B*M][prev_tiles B][tile base B*M][block queue B*M]
+//   [tile descriptors 2*B*TPS][items 16*max_items][comb 4*max_comb]
+// The items array holds the global queue's items followed by the items of the eight XCD queues.
 // Tile descriptors: for each sequence, the 64-key tiles of blocks 0..M-2 in order, as (token index of
 // the tile's first key, number of real keys); TPS = (M-1) * ceil(H/64) slots per sequence.
-// Work is handed out through 9 queues.  Queue 8 holds the query-block items (the long ones, with no
-// locality preference: they read every key); every workgroup drains it first.  Queues 0..7 belong
-// to the 8 XCDs: all query tiles of one (sequence, block) go to one queue, so the block's K/V for all
-// heads are fetched into one XCD's L2 only.  The items array is grouped by queue (queue g's items
+// Work is handed out through 9 queues.  Queues 0..7 belong to the 8 XCDs: all query tiles of one (sequence,
+// block) go to one queue, so the block's K/V for all heads are fetched into one XCD's L2 only; the query
+// block's key walk is cut where the blocks it reads change from one XCD's run to the next, and every piece is
+// put at the front of the queue of the XCD whose L2 holds those blocks (the long items go first, and the K/V
+// they walk over are the ones that XCD's other items fetch anyway).  Queue 8, drained first by every workgroup,
+// holds what has no such preference: the items of sequences that are one block only.  The items array is grouped by queue (queue g's items
 // start at QOFF[g]); a ticket t of queue g is (item QOFF[g] + t / NHG, head group t % NHG):
 // consecutive tickets cover all kv heads, which keeps every L2 channel busy.
 #define BR_PLAN_HDR 96
@@ -90,8 +91,10 @@ __host__ __device__ inline size_t br_plan_off_start() { return BR_PLAN_HDR; }
 __host__ __device__ inline size_t br_plan_off_len(int B, int M) { return BR_PLAN_HDR + (size_t)B * M; }
 __host__ __device__ inline size_t br_plan_off_tok(int B, int M) { return BR_PLAN_HDR + 2 * (size_t)B * M; }
 __host__ __device__ inline size_t br_plan_off_prev(int B, int M) { return BR_PLAN_HDR + 3 * (size_t)B * M; }
-__host__ __device__ inline int br_split_pool(int par) {
-    const int n = par / 4 + 2;
+// par / 4 pieces to fill the grid with, plus room for the cuts at the XCD queues' boundaries (up to eight per query
+// tile of a sequence that is spread over all XCDs; nhg: head groups, each of which has its own set of slots).
+__host__ __device__ inline int br_split_pool(int par, int nhg) {
+    const int n = par / 4 + 2 + 128 / (nhg > 0 ? nhg : 1);
     return n > BR_SPLIT_POOL_MAX ? BR_SPLIT_POOL_MAX : n;
 }
 __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
@@ -103,7 +106,8 @@ __host__ __device__ inline int br_plan_max_items(int B, int M, int H, int T) {
 __host__ __device__ inline int br_plan_max_comb(int B) { return BR_SPLIT_POOL_MAX / 2; }
 __host__ __device__ inline int br_plan_tps(int M, int H) { return (M > 1 ? M - 1 : 0) * ((H + BR_BN - 1) / BR_BN); }
 __host__ __device__ inline size_t br_plan_off_tbase(int B, int M) { return BR_PLAN_HDR + 3 * (size_t)B * M + (size_t)B; }
-__host__ __device__ inline size_t br_plan_off_tiles(int B, int M) { return (br_plan_off_tbase(B, M) + (size_t)B * M + 1) & ~(size_t)1; }
+__host__ __device__ inline size_t br_plan_off_bq(int B, int M) { return br_plan_off_tbase(B, M) + (size_t)B * M; }
+__host__ __device__ inline size_t br_plan_off_tiles(int B, int M) { return (br_plan_off_bq(B, M) + (size_t)B * M + 1) & ~(size_t)1; }
 __host__ __device__ inline size_t br_plan_off_items(int B, int M, int H, int T) {
     size_t o = br_plan_off_tiles(B, M) + 2 * (size_t)B * br_plan_tps(M, H);
     return (o + 15) & ~(size_t)15;   // 64-byte aligned items

@@ -73,7 +73,7 @@ __device__ inline int splits_for(int ntiles, int chunk) {
 }
 
 // par: workgroups of the prefill grid per head group, i.e. how many of a plan's items run side by side.
-// pool: split-KV partial slots the caller's workspace has room for (br_split_pool(par)).
+// pool: split-KV partial slots the caller's workspace has room for (br_split_pool).
 __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__ plan, int B, int M, int H, int T, int packed, int par, int pool) {
     __shared__ int sh[kPlanThreads / 64];
     __shared__ int s_bad;
@@ -136,64 +136,153 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     __syncthreads();
 
     // Work distribution.
-    // The query-block items (long walks, split) form the global queue, drained first.  All other items keep
-    // their natural order (sequence, block, query tile) and that list is cut into eight contiguous runs of
-    // equal estimated work, one per XCD queue: an XCD then works on a few adjacent blocks at a time (their
-    // K/V stay in its L2), and the runs end together, so that no workgroup has to go looking for work in other
-    // queues at the end of the kernel (polling the ticket counters there slows the memory accesses of every
-    // workgroup still working).  Estimated work of an item: its key tiles plus a constant for set-up and
-    // epilogue.
+    // All items but the query blocks' keep their natural order (sequence, block, query tile) and that list is cut
+    // into eight contiguous runs of equal estimated work, one per XCD queue: an XCD then works on a few adjacent
+    // blocks at a time (their K/V stay in its L2), and the runs end together, so that no workgroup has to go looking
+    // for work in other queues at the end of the kernel (polling the ticket counters there slows the memory accesses
+    // of every workgroup still working).  Estimated work of an item: its key tiles plus a constant for set-up and
+    // epilogue.  A query block reads the K/V of every earlier block of its sequence: its key walk is cut where those
+    // blocks pass from one XCD's run to the next and each stretch is handed to that XCD (at the front of its queue:
+    // long items first), so that the walk finds the tiles in the L2 that the blocks' own items fill anyway instead of
+    // pulling all K/V of the sequence into a second L2.
     constexpr int kItemOverhead = 2;
     auto item_weight = [&](int nprev_t, int tt, int L) {
         int e = (tt + 1) * T < L ? (tt + 1) * T : L;
         return nprev_t + ceil_div(e, BR_BN) + kItemOverhead;
     };
+    int* bq = plan + br_plan_off_bq(B, M);
     __shared__ int s_qfirst[8];
+    __shared__ int s_base[BR_NQUEUES], s_nsplit[BR_NQUEUES];
     if (tid < 8) s_qfirst[tid] = 0x7fffffff;
     __syncthreads();
 
-    // Length of a split of the query block's key walk.  The walk is cut so that the batch has enough items to fill
-    // the grid, and no further: every split costs a set-up, an epilogue and a set of partials to write and merge,
-    // while a long split still ends with the others because the split items are handed out first.  So: the estimated
-    // work per workgroup (all items' key tiles plus their constant, over the workgroups that run side by side) less
-    // one ordinary item - the workgroup that takes a split still has to fit one of those before the kernel ends, which
-    // is what decides at a batch of one - and at least BR_MIN_CHUNK.
+    // Ordinary (not query-block) items of the pair p = (b, m): how many, their weight, the prefix tiles they walk.
+    auto ordinary = [&](int p, int& nq, int& npt, int& L) -> int {
+        nq = 0; npt = 0; L = 0;
+        if (p >= BM) return 0;
+        const int b = p / M, m = p - b * M;
+        if (m == M - 1) return 0;
+        L = len[p];
+        nq = ceil_div(L, T);
+        npt = br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0;
+        int w = 0;
+        for (int tt = 0; tt < nq; ++tt) w += item_weight(npt, tt, L);
+        return w;
+    };
+
+    // Totals: all items' weight (with the query blocks'), the ordinary items' weight and number.
     long long w_all = 0, w_ord = 0;
     int n_ord = 0;
     for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
         const int p = p0 + tid;
-        int w = 0, nq = 0;
-        bool last = false;
-        if (p < BM) {
-            const int b = p / M, m = p - b * M;
-            const int L = len[p];
-            nq = ceil_div(L, T);
-            last = m == M - 1;
-            const int np = last ? (M > 1 ? prev_tiles[b] : 0) : (br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0);
-            for (int tt = 0; tt < nq; ++tt) w += item_weight(np, tt, L);
+        int nq, npt, L;
+        int w = ordinary(p, nq, npt, L), wq = 0;
+        if (p < BM && p % M == M - 1) {
+            const int b = p / M, Lq = len[p], pt = M > 1 ? prev_tiles[b] : 0;
+            for (int tt = 0; tt * T < Lq; ++tt) wq += item_weight(pt, tt, Lq);
         }
         int tot;
-        block_exclusive_scan(w, sh, &tot);
+        block_exclusive_scan(w + wq, sh, &tot);
         w_all += tot;
-        block_exclusive_scan(last ? 0 : w, sh, &tot);
+        block_exclusive_scan(w, sh, &tot);
         w_ord += tot;
-        block_exclusive_scan(last ? 0 : nq, sh, &tot);
+        block_exclusive_scan(nq, sh, &tot);
         n_ord += tot;
     }
+    const long long w_total = w_ord;
+
+    // Queue of every ordinary item (by the weight before it), first item of every queue, queue of every block (that of
+    // its first item).
+    {
+        int base_x = 0;
+        long long base_w = 0;
+        for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
+            const int p = p0 + tid;
+            int nq, npt, L;
+            const int w = ordinary(p, nq, npt, L);
+            int tot;
+            const int off_x = base_x + block_exclusive_scan(nq, sh, &tot);
+            base_x += tot;
+            long long off_w = base_w + block_exclusive_scan(w, sh, &tot);
+            base_w += tot;
+            if (p < BM) bq[p] = -1;
+            for (int k = 0; k < nq; ++k) {
+                int q = w_total > 0 ? (int)(off_w * 8 / w_total) : 0;
+                q = q > 7 ? 7 : q;
+                if (k == 0) bq[p] = q;
+                atomicMin(&s_qfirst[q], off_x + k);
+                off_w += item_weight(npt, nq - 1 - k, L);
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        // a queue that received no item starts where the next one starts
+        int nxt = n_ord;
+        for (int g = 7; g >= 0; --g) {
+            if (s_qfirst[g] == 0x7fffffff) s_qfirst[g] = nxt;
+            nxt = s_qfirst[g];
+        }
+    }
+    __syncthreads();
+
+    // The pieces of the key walk of query tile tt of sequence b's query block, in walk order: fn(index, first tile,
+    // tiles, queue).  The earlier blocks' tiles are cut where the blocks' queue changes (a stretch shorter than
+    // min_seg tiles stays with the next one), the query block's own tiles go with the last stretch, and every
+    // stretch is cut into pieces of at most `chunk` tiles.  Returns the number of pieces.
+    auto walk_pieces = [&](int b, int tt, int chunk, int min_seg, auto&& fn) -> int {
+        const int L = len[b * M + M - 1];
+        const int e = (tt + 1) * T < L ? (tt + 1) * T : L;
+        const int nself = ceil_div(e, BR_BN);
+        int count = 0;
+        auto close = [&](int lo, int n, int q) {
+            int parts = ceil_div(n, chunk);
+            parts = parts < 1 ? 1 : parts;
+            for (int s = 0; s < parts; ++s) {
+                const int a = lo + (int)((long long)s * n / parts), z = lo + (int)((long long)(s + 1) * n / parts);
+                fn(count, a, z - a, q);
+                ++count;
+            }
+        };
+        int seg_lo = 0, seg_n = 0, seg_q = -1;
+        for (int m = 0; m < M - 1; ++m) {
+            const int nt = ceil_div(len[b * M + m], BR_BN);
+            if (nt == 0) continue;
+            const int q = bq[b * M + m];
+            if (seg_q >= 0 && q != seg_q && seg_n >= min_seg) {
+                close(seg_lo, seg_n, seg_q);
+                seg_lo += seg_n;
+                seg_n = 0;
+                seg_q = q;
+            }
+            if (seg_q < 0) seg_q = q;
+            seg_n += nt;
+        }
+        close(seg_lo, seg_n + nself, seg_q < 0 ? BR_GLOBAL_QUEUE : seg_q);
+        return count;
+    };
+    auto no_op = [](int, int, int, int) {};
+
+    // Length of a piece.  The walks are cut so that the batch has enough items to fill the grid, and no further: every
+    // piece costs a set-up, an epilogue and a set of partials to write and merge, while a long piece still ends with the
+    // others because the pieces are handed out first.  So: the estimated work per workgroup (all items' key tiles plus
+    // their constant, over the workgroups that run side by side) less one ordinary item - the workgroup that takes a
+    // piece still has to fit one of those before the kernel ends, which is what decides at a batch of one - and at
+    // least BR_MIN_CHUNK; and long enough that the batch's pieces fit the pool of partial slots: lengthen until they
+    // do, and where longer pieces no longer help (what remains are the cuts between XCDs) join short stretches to
+    // their neighbours; with both beyond every walk's length nothing is split at all, so this ends.
     int chunk = (int)(w_all / (par > 0 ? par : 1)) - (n_ord > 0 ? (int)(w_ord / n_ord) : 0);
     chunk = chunk < BR_MIN_CHUNK ? BR_MIN_CHUNK : chunk;
-    // ... and long enough that the batch's splits fit the pool of partial slots: lengthen until they do (a chunk
-    // longer than every walk means no split at all, so this ends)
+    int min_seg = BR_MIN_CHUNK, need_before = 0x7fffffff;
     for (;;) {
         int need = 0;
         for (int b0 = 0; b0 < B; b0 += kPlanThreads) {
             const int b = b0 + tid;
             int mine = 0;
             if (b < B) {
-                const int L = len[b * M + M - 1], pt = M > 1 ? prev_tiles[b] : 0;
+                const int L = len[b * M + M - 1];
                 for (int tt = 0; tt * T < L; ++tt) {
-                    const int e = (tt + 1) * T < L ? (tt + 1) * T : L;
-                    const int ns = splits_for(pt + ceil_div(e, BR_BN), chunk);
+                    const int ns = walk_pieces(b, tt, chunk, min_seg, no_op);
                     mine += ns > 1 ? ns : 0;
                 }
             }
@@ -202,140 +291,46 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             need += tot;
         }
         if (need <= pool) break;
-        chunk += (chunk + 1) / 2;
+        if (need >= need_before) min_seg *= 2;
+        need_before = need;
+        if (chunk < (1 << 24)) chunk += (chunk + 1) / 2;
     }
 
-    struct Counts {
-        int glob, x, w, comb, slots;
-    };
-    // what one (sequence, block) pair contributes; pairs are visited sequence by sequence, the query block first
-    auto count_pair = [&](int p, Counts& c, int& b, int& m, int& L, int& nq, int& pt, int& npt, bool& is_last) {
-        c = Counts{0, 0, 0, 0, 0};
-        b = p / M;
-        const int jj = p - b * M;
-        m = jj == 0 ? M - 1 : jj - 1;
-        is_last = jj == 0;
-        L = len[b * M + m];
-        nq = ceil_div(L, T);
-        if (is_last) {
-            pt = M > 1 ? prev_tiles[b] : 0;
-            for (int tt = 0; tt < nq; ++tt) {
-                int e = (tt + 1) * T < L ? (tt + 1) * T : L;
-                int ns = splits_for(pt + ceil_div(e, BR_BN), chunk);
-                c.glob += ns;
-                c.comb += ns > 1;
-                c.slots += ns > 1 ? ns : 0;
-            }
-        } else {
-            c.x = nq;
-            npt = br_prev_blocks(m, M) > 0 ? ceil_div(len[b * M], BR_BN) : 0;
-            for (int tt = 0; tt < nq; ++tt) c.w += item_weight(npt, tt, L);
+    // Layout of the items array: [global queue][queue 0: its pieces, its ordinary items][queue 1: ...] ...
+    // One thread per sequence (the entry points admit at most kPlanThreads sequences per plan) counts the pieces of its
+    // query block per queue; scans give every sequence its offsets.
+    int my_cnt[BR_NQUEUES], my_off[BR_NQUEUES], my_comb = 0, my_slots = 0;
+    for (int q = 0; q < BR_NQUEUES; ++q) my_cnt[q] = 0;
+    if (tid < B) {
+        const int L = len[tid * M + M - 1];
+        for (int tt = 0; tt * T < L; ++tt) {
+            const int ns = walk_pieces(tid, tt, chunk, min_seg, [&](int, int, int, int q) { ++my_cnt[q]; });
+            my_comb += ns > 1;
+            my_slots += ns > 1 ? ns : 0;
         }
-    };
-
-    // Pass 1: totals.
-    int n_glob_total = 0, n_x_total = 0, n_comb_total = 0;
-    long long w_total = 0;
-    for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
-        const int p = p0 + tid;
-        Counts c = Counts{0, 0, 0, 0, 0};
-        if (p < BM) {
-            int b, m, L, nq, pt, npt;
-            bool is_last;
-            count_pair(p, c, b, m, L, nq, pt, npt, is_last);
-        }
+    }
+    int n_comb_total = 0, n_slot_total = 0;
+    for (int q = 0; q < BR_NQUEUES; ++q) {
         int tot;
-        block_exclusive_scan(c.glob, sh, &tot);
-        n_glob_total += tot;
-        block_exclusive_scan(c.x, sh, &tot);
-        n_x_total += tot;
-        block_exclusive_scan(c.w, sh, &tot);
-        w_total += tot;
-        block_exclusive_scan(c.comb, sh, &tot);
-        n_comb_total += tot;
+        my_off[q] = block_exclusive_scan(my_cnt[q], sh, &tot);
+        if (tid == 0) s_nsplit[q] = tot;
     }
-
-    // Pass 2: the items array is [global queue][XCD queues].
-    const int xoff = n_glob_total;
-    int base_glob = 0, base_x = xoff, base_comb = 0, base_slot = 0;
-    long long base_w = 0;
-    for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
-        const int p = p0 + tid;
-        Counts c = Counts{0, 0, 0, 0, 0};
-        int b = 0, m = 0, L = 0, nq = 0, pt = 0, npt = 0;
-        bool is_last = false;
-        if (p < BM) count_pair(p, c, b, m, L, nq, pt, npt, is_last);
-        int tot;
-        int off_g = base_glob + block_exclusive_scan(c.glob, sh, &tot);
-        base_glob += tot;
-        const int off_x = base_x + block_exclusive_scan(c.x, sh, &tot);
-        base_x += tot;
-        int off_c = base_comb + block_exclusive_scan(c.comb, sh, &tot);
-        base_comb += tot;
-        const int off_s = base_slot + block_exclusive_scan(c.slots, sh, &tot);
-        base_slot += tot;
-        long long off_w = base_w + block_exclusive_scan(c.w, sh, &tot);
-        base_w += tot;
-        if (p < BM) {
-            const int pe = br_prev_blocks(m, M);
-            BrItem it;
-            it.b = b; it.m = m; it.pe = pe;
-            it.len_m = L; it.start_m = start[b * M + m]; it.len0 = len[b * M]; it.start0 = start[b * M];
-            it.tok_m = tok[b * M + m]; it.tok0 = tok[b * M];
-            it.pad[0] = it.pad[1] = 0;
-            if (!is_last) {
-                it.nprev = npt;
-                // a block's query tiles are handed out from the last (the longest walk) to the first: what a queue
-                // ends on are short items
-                for (int k = 0; k < nq; ++k) {
-                    const int tt = nq - 1 - k;
-                    it.t0 = tt * T; it.f_lo = 0;
-                    it.ntiles = 0x7fffffff; it.slot = -1;
-                    items[off_x + k] = it;
-                    int q = w_total > 0 ? (int)(off_w * 8 / w_total) : 0;
-                    q = q > 7 ? 7 : q;
-                    atomicMin(&s_qfirst[q], off_x + k);
-                    off_w += item_weight(npt, tt, L);
-                }
-            } else {
-                it.nprev = pt;
-                int slot = off_s;                            // slots of the batch's pool, in item order
-                for (int tt = 0; tt < nq; ++tt) {
-                    int e = (tt + 1) * T < L ? (tt + 1) * T : L;
-                    int nself = ceil_div(e, BR_BN);
-                    int nt = pt + nself;
-                    int ns = splits_for(nt, chunk);
-                    if (ns > 1) {
-                        BrComb cb;
-                        cb.b = b; cb.t0 = tt * T; cb.slot0 = slot; cb.nsplit = ns;
-                        comb[off_c++] = cb;
-                    }
-                    for (int s = 0; s < ns; ++s) {
-                        int lo = (int)((long long)s * nt / ns);
-                        int hi = (int)((long long)(s + 1) * nt / ns);
-                        it.t0 = tt * T; it.f_lo = lo;
-                        it.ntiles = ns > 1 ? hi - lo : 0x7fffffff; it.slot = ns > 1 ? slot + s : -1;
-                        items[off_g++] = it;
-                    }
-                    if (ns > 1) slot += ns;
-                }
-            }
-        }
-    }
+    const int off_comb = block_exclusive_scan(my_comb, sh, &n_comb_total);
+    const int off_slot = block_exclusive_scan(my_slots, sh, &n_slot_total);
     __syncthreads();
     if (tid == 0) {
-        // a queue that received no item starts where the next one starts
-        int nxt = xoff + n_x_total;
-        for (int g = 7; g >= 0; --g) {
-            int f = s_qfirst[g];
-            if (f == 0x7fffffff) f = nxt;
-            hdr[BR_PH_QOFF + g] = f;
-            hdr[BR_PH_QCOUNT + g] = nxt - f;
-            nxt = f;
+        int nxt = s_nsplit[BR_GLOBAL_QUEUE];
+        for (int g = 0; g < 8; ++g) {
+            s_base[g] = nxt;
+            const int ord = (g < 7 ? s_qfirst[g + 1] : n_ord) - s_qfirst[g];
+            hdr[BR_PH_QOFF + g] = nxt;
+            hdr[BR_PH_QCOUNT + g] = s_nsplit[g] + ord;
+            nxt += s_nsplit[g] + ord;
         }
+        s_base[BR_GLOBAL_QUEUE] = 0;
         hdr[BR_PH_QOFF + BR_GLOBAL_QUEUE] = 0;
-        hdr[BR_PH_QCOUNT + BR_GLOBAL_QUEUE] = n_glob_total;
-        hdr[BR_PH_NITEMS] = xoff + n_x_total;
+        hdr[BR_PH_QCOUNT + BR_GLOBAL_QUEUE] = s_nsplit[BR_GLOBAL_QUEUE];
+        hdr[BR_PH_NITEMS] = nxt;
         hdr[BR_PH_NCOMB] = n_comb_total;
         hdr[BR_PH_PACKED] = packed;
         hdr[BR_PH_NONCONTIG] = s_bad;
@@ -343,7 +338,75 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         hdr[BR_PH_MAX_COMB] = br_plan_max_comb(B);
         hdr[BR_PH_T] = T;
         hdr[BR_PH_POOL] = pool;
-        hdr[BR_PH_NSLOTS] = base_slot;
+        hdr[BR_PH_NSLOTS] = n_slot_total;
+    }
+    __syncthreads();
+
+    // Ordinary items: queue g's start at s_base[g] + its pieces, in their natural order.
+    {
+        int base_x = 0;
+        long long base_w = 0;
+        for (int p0 = 0; p0 < BM; p0 += kPlanThreads) {
+            const int p = p0 + tid;
+            int nq, npt, L;
+            const int w = ordinary(p, nq, npt, L);
+            int tot;
+            const int off_x = base_x + block_exclusive_scan(nq, sh, &tot);
+            base_x += tot;
+            long long off_w = base_w + block_exclusive_scan(w, sh, &tot);
+            base_w += tot;
+            if (nq > 0) {
+                const int b = p / M, m = p - b * M;
+                BrItem it;
+                it.b = b; it.m = m; it.pe = br_prev_blocks(m, M);
+                it.len_m = L; it.start_m = start[p]; it.len0 = len[b * M]; it.start0 = start[b * M];
+                it.tok_m = tok[p]; it.tok0 = tok[b * M];
+                it.pad[0] = it.pad[1] = 0;
+                it.nprev = npt;
+                it.f_lo = 0; it.ntiles = 0x7fffffff; it.slot = -1;
+                // a block's query tiles are handed out from the last (the longest walk) to the first: what a queue
+                // ends on are short items
+                for (int k = 0; k < nq; ++k) {
+                    const int tt = nq - 1 - k;
+                    int q = w_total > 0 ? (int)(off_w * 8 / w_total) : 0;
+                    q = q > 7 ? 7 : q;
+                    it.t0 = tt * T;
+                    items[s_base[q] + s_nsplit[q] + (off_x + k - s_qfirst[q])] = it;
+                    off_w += item_weight(npt, tt, L);
+                }
+            }
+        }
+    }
+    // The query blocks' pieces (one thread per sequence; the offsets of the counting round above).
+    if (tid < B) {
+        const int b = tid;
+        const int pq = b * M + M - 1;
+        const int L = len[pq];
+        BrItem it;
+        it.b = b; it.m = M - 1; it.pe = br_prev_blocks(M - 1, M);
+        it.len_m = L; it.start_m = start[pq]; it.len0 = len[b * M]; it.start0 = start[b * M];
+        it.tok_m = tok[pq]; it.tok0 = tok[b * M];
+        it.pad[0] = it.pad[1] = 0;
+        it.nprev = M > 1 ? prev_tiles[b] : 0;
+        int pos[BR_NQUEUES];
+        for (int q = 0; q < BR_NQUEUES; ++q) pos[q] = s_base[q] + my_off[q];
+        int slot = off_slot, ci = off_comb;
+        for (int tt = 0; tt * T < L; ++tt) {
+            const int ns = walk_pieces(b, tt, chunk, min_seg, no_op);
+            if (ns > 1) {
+                BrComb cb;
+                cb.b = b; cb.t0 = tt * T; cb.slot0 = slot; cb.nsplit = ns;
+                comb[ci++] = cb;
+            }
+            it.t0 = tt * T;
+            walk_pieces(b, tt, chunk, min_seg, [&](int i, int lo, int n, int q) {
+                it.f_lo = lo;
+                it.ntiles = ns > 1 ? n : 0x7fffffff;
+                it.slot = ns > 1 ? slot + i : -1;
+                items[pos[q]++] = it;
+            });
+            if (ns > 1) slot += ns;
+        }
     }
 }
 

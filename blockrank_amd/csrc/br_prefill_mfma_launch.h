@@ -1,7 +1,7 @@
 // Instances and launcher of the block-sparse prefill kernel for one 16-bit element type (the templates live in
-// br_prefill_mfma_impl.h and br_prefill_narrow_impl.h).  The including file defines BR_LAUNCH_PREFILL, the
-// launcher's name, and, for fp16, BR_E16 / BR_E16_IS_F16.
-#include "br_prefill_narrow_impl.h"
+// br_prefill_mfma_impl.h).  The including file defines BR_LAUNCH_PREFILL, the launcher's name, and, for fp16,
+// BR_E16 / BR_E16_IS_F16.
+#include "br_prefill_mfma_impl.h"
 
 namespace {
 
@@ -17,23 +17,14 @@ void launch(const BrPrefillParams& p, int grid, hipStream_t stream) {
 
 }  // namespace
 
-// wave_rows: 16 selects the narrow-wave kernel (16 query rows per wave, 8 waves) where it exists - head dim 128, a
-// geometry of four 32-row blocks per query tile, no rotary tables -, anything else the 32-row kernel.
 // Returns 0 on success, -1 if (D, NW) has no instantiation, 1 if the score reduction asked for with ``rank`` does not
 // fit (nothing is launched in either case).
 int BR_LAUNCH_PREFILL(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
-                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank, int wave_rows) {
+                           hipEvent_t ev_start, hipEvent_t ev_stop, const BrTileScoreParams* rank) {
     const int per_cu = NW <= 4 ? 2 : 1;
     const int grid = n_cu * per_cu;
     if (rank && (size_t)(rank->M - 2) * sizeof(float) > 60 * 1024) return 1;
     if (ev_start) (void)hipEventRecord(ev_start, stream);
-    if (wave_rows == 16 && D == 128 && NW == 4 && p.rope_cos == nullptr) {
-        if (p.score_part != nullptr || p.lse != nullptr)
-            hipLaunchKernelGGL((br_prefill_narrow_kernel<128, true>), dim3(grid), dim3(512), 0, stream, p);
-        else
-            hipLaunchKernelGGL((br_prefill_narrow_kernel<128, false>), dim3(grid), dim3(512), 0, stream, p);
-        goto launched;
-    }
 #define BR_CASE(DD, WW)                                   \
     if (D == DD && NW == WW) {                            \
         launch<DD, WW>(p, grid, stream);                  \

@@ -75,7 +75,7 @@ int br_plan_build_packed(const int32_t* lens, int B, int M, int H, int Nq, int N
 /* Bytes of scratch br_prefill_fwd needs: the split-KV partials of the query blocks' key walks.  The plan cuts those
  * walks only as far as it takes to give every workgroup of the grid work, and takes the slots from one pool for the
  * whole batch, so the size follows from the head layout and the current device's compute-unit count and does not grow
- * with B (about 10 MB for 32 / 8 heads of dim 128 on 256 compute units).  0 without a HIP device. */
+ * with B (about 18 MB for 32 / 8 heads of dim 128 on 256 compute units).  0 without a HIP device. */
 size_t br_prefill_workspace_bytes(int B, int Nq, int Nkv, int D);
 
 /* Block-sparse prefill attention.  Replaces sdpa_blockrank_attention_forward /
@@ -110,7 +110,7 @@ int br_prefill_fwd_events(const void* q, const void* k, const void* v, void* out
  * library's code object, which is when the runtime sets the array up), and every request needs a plan, so by the
  * time this entry runs - under graph capture too - the address is known.
  * A request whose br_prefill_workspace_bytes() exceeds that size is refused with BR_ERR_SPACE (no head layout
- * of a current model does: 32 / 8 heads of dim 128 need about 10 MB whatever the batch).  Every call on a GPU
+ * of a current model does: 32 / 8 heads of dim 128 need about 18 MB whatever the batch).  Every call on a GPU
  * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream,
  * one after the other, do not.  Nothing in the array has to be cleared between calls (a call reads only the
  * partials it wrote itself). */

@@ -44,7 +44,7 @@ def test_pure_host_entry_points():
     # the split partials' pool follows the head layout and the device's compute units, not the batch (0: no device here)
     ws = lib.br_prefill_workspace_bytes(4, 32, 8, 128)
     assert ws == lib.br_prefill_workspace_bytes(64, 32, 8, 128)
-    assert ws == 0 or 4 << 20 < ws < 16 << 20
+    assert ws == 0 or 4 << 20 < ws < 32 << 20
     assert lib.br_doc_scores_workspace_bytes(4, 32, 22, 2) == 4 * 32 * 2 * 20 * 2 * 4
     assert ws == 0 or lib.br_prefill_fp8qk_workspace_bytes(4, 32, 8, 128, 22, 4 * 3520) > ws
     # backward: fp32 sums of the query block's dQ rows and of the prefix keys' dK / dV, rounded up to 256 bytes, then one
