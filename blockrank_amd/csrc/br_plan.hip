@@ -9,7 +9,7 @@
 
 namespace {
 
-constexpr int kPlanThreads = 1024;
+constexpr int kPlanThreads = 512;
 
 // One wave per block: count real tokens, find the first and the last.  len is written negated
 // (-1 - count) when the real tokens are not one contiguous span; the plan kernel repairs the sign
@@ -64,6 +64,36 @@ __device__ int block_exclusive_scan(int x, int* sh, int* total) {
     __syncthreads();
     *total = tot;
     return base + incl - x;
+}
+
+// The same for N values per thread at once (one pair of barriers for all of them): x[i] becomes the exclusive
+// prefix of x[i] over the workgroup, tot[i] the total.
+template <int N>
+__device__ void block_exclusive_scan_n(int (&x)[N], int (&tot)[N], int* shn /* N * kPlanThreads / 64 ints */) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int incl[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        incl[i] = x[i];
+        for (int o = 1; o < 64; o <<= 1) {
+            int y = __shfl_up(incl[i], o);
+            if (lane >= o) incl[i] += y;
+        }
+        if (lane == 63) shn[i * (kPlanThreads / 64) + wave] = incl[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        int base = 0, t = 0;
+        for (int w = 0; w < kPlanThreads / 64; ++w) {
+            const int v = shn[i * (kPlanThreads / 64) + w];
+            if (w < wave) base += v;
+            t += v;
+        }
+        tot[i] = t;
+        x[i] = base + incl[i] - x[i];
+    }
+    __syncthreads();
 }
 
 // Split count for a query tile of the query block: enough splits that each covers about ``chunk`` key tiles.
@@ -226,11 +256,64 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     }
     __syncthreads();
 
+    // What the walks below read about every block - its key tiles and its queue - staged in LDS once: a walk is a
+    // serial loop over a sequence's blocks run by a single thread, and from global memory every step of it is a
+    // round trip of its own.
+    constexpr int kStage = 8192;
+    __shared__ unsigned short s_nt[kStage];
+    __shared__ signed char s_bq[kStage];
+    const bool staged = BM <= kStage;
+    if (staged) {
+        for (int p = tid; p < BM; p += kPlanThreads) {
+            const int nt = ceil_div(len[p], BR_BN);
+            s_nt[p] = (unsigned short)(nt > 0xffff ? 0xffff : nt);
+            s_bq[p] = (signed char)bq[p];
+        }
+    }
+    __syncthreads();
+    auto blk_tiles = [&](int p) -> int { return staged ? (int)s_nt[p] : ceil_div(len[p], BR_BN); };
+    auto blk_queue = [&](int p) -> int { return staged ? (int)s_bq[p] : bq[p]; };
+
+    // The stretches of a sequence's earlier blocks that one XCD's queue owns: first tile, tiles, queue.  The queues
+    // follow the blocks' order, so there are at most eight; a stretch shorter than min_seg tiles stays with the next
+    // one.  (Small fixed arrays indexed through unrolled loops: they live in registers - a dynamically indexed local
+    // array is scratch memory, a round trip of microseconds per access for the single thread that walks a sequence.)
+    struct Segs {
+        int n;
+        int lo[8], cnt[8], q[8];
+    };
+    auto build_segs = [&](int b, int min_seg, Segs& S) {
+        S.n = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) S.lo[i] = S.cnt[i] = S.q[i] = 0;
+        int seg_lo = 0, seg_n = 0, seg_q = -1;
+        auto push = [&]() {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (i == S.n) {
+                    S.lo[i] = seg_lo; S.cnt[i] = seg_n; S.q[i] = seg_q;
+                }
+            ++S.n;
+        };
+        for (int m = 0; m < M - 1; ++m) {
+            const int nt = blk_tiles(b * M + m);
+            if (nt == 0) continue;
+            const int q = blk_queue(b * M + m);
+            if (seg_q >= 0 && q != seg_q && seg_n >= min_seg && S.n < 7) {
+                push();
+                seg_lo += seg_n;
+                seg_n = 0;
+                seg_q = q;
+            }
+            if (seg_q < 0) seg_q = q;
+            seg_n += nt;
+        }
+        if (seg_q >= 0) push();
+    };
     // The pieces of the key walk of query tile tt of sequence b's query block, in walk order: fn(index, first tile,
-    // tiles, queue).  The earlier blocks' tiles are cut where the blocks' queue changes (a stretch shorter than
-    // min_seg tiles stays with the next one), the query block's own tiles go with the last stretch, and every
-    // stretch is cut into pieces of at most `chunk` tiles.  Returns the number of pieces.
-    auto walk_pieces = [&](int b, int tt, int chunk, int min_seg, auto&& fn) -> int {
+    // tiles, queue).  Every stretch is cut into pieces of at most `chunk` tiles; the query block's own tiles go with the
+    // last stretch (a sequence without earlier keys has them alone, in the global queue).  Returns the number of pieces.
+    auto walk_pieces = [&](int b, int tt, int chunk, const Segs& S, auto&& fn) -> int {
         const int L = len[b * M + M - 1];
         const int e = (tt + 1) * T < L ? (tt + 1) * T : L;
         const int nself = ceil_div(e, BR_BN);
@@ -244,24 +327,27 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
                 ++count;
             }
         };
-        int seg_lo = 0, seg_n = 0, seg_q = -1;
-        for (int m = 0; m < M - 1; ++m) {
-            const int nt = ceil_div(len[b * M + m], BR_BN);
-            if (nt == 0) continue;
-            const int q = bq[b * M + m];
-            if (seg_q >= 0 && q != seg_q && seg_n >= min_seg) {
-                close(seg_lo, seg_n, seg_q);
-                seg_lo += seg_n;
-                seg_n = 0;
-                seg_q = q;
-            }
-            if (seg_q < 0) seg_q = q;
-            seg_n += nt;
+        if (S.n == 0) {
+            close(0, nself, BR_GLOBAL_QUEUE);
+            return count;
         }
-        close(seg_lo, seg_n + nself, seg_q < 0 ? BR_GLOBAL_QUEUE : seg_q);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i < S.n) close(S.lo[i], S.cnt[i] + (i == S.n - 1 ? nself : 0), S.q[i]);
         return count;
     };
     auto no_op = [](int, int, int, int) {};
+    // a[q] += 1 for a register-resident array of the nine queues; returns the value before
+    auto bump = [](int (&a)[BR_NQUEUES], int q) -> int {
+        int r = 0;
+#pragma unroll
+        for (int i = 0; i < BR_NQUEUES; ++i)
+            if (i == q) {
+                r = a[i];
+                a[i] = r + 1;
+            }
+        return r;
+    };
 
     // Length of a piece.  The walks are cut so that the batch has enough items to fill the grid, and no further: every
     // piece costs a set-up, an epilogue and a set of partials to write and merge, while a long piece still ends with the
@@ -274,49 +360,52 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     int chunk = (int)(w_all / (par > 0 ? par : 1)) - (n_ord > 0 ? (int)(w_ord / n_ord) : 0);
     chunk = chunk < BR_MIN_CHUNK ? BR_MIN_CHUNK : chunk;
     int min_seg = BR_MIN_CHUNK, need_before = 0x7fffffff;
+    Segs segs;
+    segs.n = 0;
+    const int Lq = tid < B ? len[tid * M + M - 1] : 0;      // (one sequence per thread: the entry points admit at most kPlanThreads)
+    if (tid < B) build_segs(tid, min_seg, segs);
     for (;;) {
-        int need = 0;
-        for (int b0 = 0; b0 < B; b0 += kPlanThreads) {
-            const int b = b0 + tid;
-            int mine = 0;
-            if (b < B) {
-                const int L = len[b * M + M - 1];
-                for (int tt = 0; tt * T < L; ++tt) {
-                    const int ns = walk_pieces(b, tt, chunk, min_seg, no_op);
-                    mine += ns > 1 ? ns : 0;
-                }
-            }
-            int tot;
-            block_exclusive_scan(mine, sh, &tot);
-            need += tot;
+        int mine = 0;
+        for (int tt = 0; tt * T < Lq; ++tt) {
+            const int ns = walk_pieces(tid, tt, chunk, segs, no_op);
+            mine += ns > 1 ? ns : 0;
         }
+        int need;
+        block_exclusive_scan(mine, sh, &need);
         if (need <= pool) break;
-        if (need >= need_before) min_seg *= 2;
+        if (need >= need_before) {
+            min_seg *= 2;
+            if (tid < B) build_segs(tid, min_seg, segs);
+        }
         need_before = need;
         if (chunk < (1 << 24)) chunk += (chunk + 1) / 2;
     }
 
     // Layout of the items array: [global queue][queue 0: its pieces, its ordinary items][queue 1: ...] ...
-    // One thread per sequence (the entry points admit at most kPlanThreads sequences per plan) counts the pieces of its
-    // query block per queue; scans give every sequence its offsets.
+    // The thread of every sequence counts the pieces of its query block per queue; scans give it its offsets.
     int my_cnt[BR_NQUEUES], my_off[BR_NQUEUES], my_comb = 0, my_slots = 0;
+#pragma unroll
     for (int q = 0; q < BR_NQUEUES; ++q) my_cnt[q] = 0;
-    if (tid < B) {
-        const int L = len[tid * M + M - 1];
-        for (int tt = 0; tt * T < L; ++tt) {
-            const int ns = walk_pieces(tid, tt, chunk, min_seg, [&](int, int, int, int q) { ++my_cnt[q]; });
-            my_comb += ns > 1;
-            my_slots += ns > 1 ? ns : 0;
-        }
+    for (int tt = 0; tt * T < Lq; ++tt) {
+        const int ns = walk_pieces(tid, tt, chunk, segs, [&](int, int, int, int q) { bump(my_cnt, q); });
+        my_comb += ns > 1;
+        my_slots += ns > 1 ? ns : 0;
     }
-    int n_comb_total = 0, n_slot_total = 0;
+    // (all eleven counts through one scan)
+    __shared__ int s_scan[(BR_NQUEUES + 2) * (kPlanThreads / 64)];
+    int sc[BR_NQUEUES + 2], sc_tot[BR_NQUEUES + 2];
+#pragma unroll
+    for (int q = 0; q < BR_NQUEUES; ++q) sc[q] = my_cnt[q];
+    sc[BR_NQUEUES] = my_comb;
+    sc[BR_NQUEUES + 1] = my_slots;
+    block_exclusive_scan_n<BR_NQUEUES + 2>(sc, sc_tot, s_scan);
+#pragma unroll
     for (int q = 0; q < BR_NQUEUES; ++q) {
-        int tot;
-        my_off[q] = block_exclusive_scan(my_cnt[q], sh, &tot);
-        if (tid == 0) s_nsplit[q] = tot;
+        my_off[q] = sc[q];
+        if (tid == 0) s_nsplit[q] = sc_tot[q];
     }
-    const int off_comb = block_exclusive_scan(my_comb, sh, &n_comb_total);
-    const int off_slot = block_exclusive_scan(my_slots, sh, &n_slot_total);
+    const int off_comb = sc[BR_NQUEUES], off_slot = sc[BR_NQUEUES + 1];
+    const int n_comb_total = sc_tot[BR_NQUEUES], n_slot_total = sc_tot[BR_NQUEUES + 1];
     __syncthreads();
     if (tid == 0) {
         int nxt = s_nsplit[BR_GLOBAL_QUEUE];
@@ -377,7 +466,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             }
         }
     }
-    // The query blocks' pieces (one thread per sequence; the offsets of the counting round above).
+    // The query blocks' pieces (the thread of every sequence; the offsets of the counting pass above).
     if (tid < B) {
         const int b = tid;
         const int pq = b * M + M - 1;
@@ -389,21 +478,22 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
         it.pad[0] = it.pad[1] = 0;
         it.nprev = M > 1 ? prev_tiles[b] : 0;
         int pos[BR_NQUEUES];
+#pragma unroll
         for (int q = 0; q < BR_NQUEUES; ++q) pos[q] = s_base[q] + my_off[q];
         int slot = off_slot, ci = off_comb;
         for (int tt = 0; tt * T < L; ++tt) {
-            const int ns = walk_pieces(b, tt, chunk, min_seg, no_op);
+            const int ns = walk_pieces(b, tt, chunk, segs, no_op);
             if (ns > 1) {
                 BrComb cb;
                 cb.b = b; cb.t0 = tt * T; cb.slot0 = slot; cb.nsplit = ns;
                 comb[ci++] = cb;
             }
             it.t0 = tt * T;
-            walk_pieces(b, tt, chunk, min_seg, [&](int i, int lo, int n, int q) {
+            walk_pieces(b, tt, chunk, segs, [&](int i, int lo, int n, int q) {
                 it.f_lo = lo;
                 it.ntiles = ns > 1 ? n : 0x7fffffff;
                 it.slot = ns > 1 ? slot + i : -1;
-                items[pos[q]++] = it;
+                items[bump(pos, q)] = it;
             });
             if (ns > 1) slot += ns;
         }
