@@ -643,10 +643,12 @@ struct Prefill {
                     else qf[c] = as_e16x8(ld16(qrow + qoff + c * 32));
                 }
             } else {
+                // a wave without rows computes no tile (nkb is 0 below): its fragments are never read, so they are
+                // only declared defined (clearing them cost every item 32 moves ahead of the branch)
 #pragma unroll
                 for (int c = 0; c < D / 16; ++c) {
-                    if constexpr (F8) qraw[c] = u32x4{0u, 0u, 0u, 0u};
-                    else qf[c] = as_e16x8(uint4{0u, 0u, 0u, 0u});
+                    if constexpr (F8) asm volatile("" : "=v"(qraw[c]));
+                    else asm volatile("" : "=v"(qf[c]));
                 }
             }
             if constexpr (DO_ROPE) {
