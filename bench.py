@@ -450,16 +450,17 @@ def main():
     if args.alias_q:
         q = q[:, :, :1].expand_as(q)
 
-    # once per forward pass: mask hook -> plan
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    if args.packed_layout:
-        mask = br.BlockMask.from_lengths(lens_dev, H=layout.H, packed=True, dtype=dtype)
-    else:
-        mask = br.blockrank_attention_mask(batch_size=layout.B, attention_mask=valid, dtype=dtype)
-    mask.plan(Nq, Nkv)
-    torch.cuda.synchronize()
-    plan_ms = (time.perf_counter() - t0) * 1e3
+    # once per forward pass: mask hook -> plan (timed on the second build: the first also loads the library's code)
+    for _ in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        if args.packed_layout:
+            mask = br.BlockMask.from_lengths(lens_dev, H=layout.H, packed=True, dtype=dtype)
+        else:
+            mask = br.blockrank_attention_mask(batch_size=layout.B, attention_mask=valid, dtype=dtype)
+        mask.plan(Nq, Nkv)
+        torch.cuda.synchronize()
+        plan_ms = (time.perf_counter() - t0) * 1e3
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
@@ -556,7 +557,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("fp8 e4m3 (Q K^T) + bf16 (P V)" if args.qk_fp8 else "bf16") if dtype == torch.bfloat16 else "f32",
+        "dtype": ("fp8 e4m3 Q K^T (power-of-two scales: one per (sequence, kv head) for K, one per row for Q; the query block's rows stay bf16) + bf16 P V"
+                  if args.qk_fp8 else "bf16") if dtype == torch.bfloat16 else "f32",
         "data": "synthetic",
         "config": {"workload": wl["desc"], "name": args.workload, "batch": layout.B, "blocks": layout.M, "block_len": layout.H,
                    "valid_tokens": layout.valid_tokens, "unmasked_pairs": pairs_n, "launch": "graph" if graph_ms is not None and graph_ms < ms_per_step else "eager",
