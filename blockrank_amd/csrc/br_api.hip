@@ -202,7 +202,7 @@ static int plan_build(const uint8_t* valid, const int32_t* lens, int left_padded
     BrGeom g16;
     int nw16;
     make_geom(Nq, Nkv, &g16, &nw16, true);                  // the shape the 16-bit forward kernels run in
-    if ((long long)br_plan_max_items(B, M, H, T) * (g16.NHG > g.NHG ? g16.NHG : g.NHG) >= (1 << 24) || B > 512)
+    if ((long long)br_plan_max_items(B, M, H, T) * (g16.NHG > g.NHG ? g16.NHG : g.NHG) >= (1 << 24))
         return fail(BR_ERR_ARG, "batch too large for one plan (B=%d, M=%d, H=%d)", B, M, H);
     const int n_cu = n_compute_units();
     if (n_cu <= 0) return fail(BR_ERR_HIP, "no HIP device");

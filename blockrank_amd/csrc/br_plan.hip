@@ -360,37 +360,49 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
     int chunk = (int)(w_all / (par > 0 ? par : 1)) - (n_ord > 0 ? (int)(w_ord / n_ord) : 0);
     chunk = chunk < BR_MIN_CHUNK ? BR_MIN_CHUNK : chunk;
     int min_seg = BR_MIN_CHUNK, need_before = 0x7fffffff;
+    // Thread tid walks the sequences tid, tid + kPlanThreads, ...  With one sequence per thread (every batch but
+    // the largest) its stretch list is built once and kept in registers; otherwise it is rebuilt at every visit.
     Segs segs;
     segs.n = 0;
-    const int Lq = tid < B ? len[tid * M + M - 1] : 0;      // (one sequence per thread: the entry points admit at most kPlanThreads)
-    if (tid < B) build_segs(tid, min_seg, segs);
+    const bool one_each = B <= kPlanThreads;
+    if (one_each && tid < B) build_segs(tid, min_seg, segs);
+    auto for_my_sequences = [&](auto&& fn) {
+        for (int b = tid; b < B; b += kPlanThreads) {
+            if (!one_each) build_segs(b, min_seg, segs);
+            fn(b, len[b * M + M - 1]);
+        }
+    };
     for (;;) {
         int mine = 0;
-        for (int tt = 0; tt * T < Lq; ++tt) {
-            const int ns = walk_pieces(tid, tt, chunk, segs, no_op);
-            mine += ns > 1 ? ns : 0;
-        }
+        for_my_sequences([&](int b, int Lq) {
+            for (int tt = 0; tt * T < Lq; ++tt) {
+                const int ns = walk_pieces(b, tt, chunk, segs, no_op);
+                mine += ns > 1 ? ns : 0;
+            }
+        });
         int need;
         block_exclusive_scan(mine, sh, &need);
         if (need <= pool) break;
         if (need >= need_before) {
             min_seg *= 2;
-            if (tid < B) build_segs(tid, min_seg, segs);
+            if (one_each && tid < B) build_segs(tid, min_seg, segs);
         }
         need_before = need;
         if (chunk < (1 << 24)) chunk += (chunk + 1) / 2;
     }
 
     // Layout of the items array: [global queue][queue 0: its pieces, its ordinary items][queue 1: ...] ...
-    // The thread of every sequence counts the pieces of its query block per queue; scans give it its offsets.
+    // Every thread counts the pieces of its sequences' query blocks per queue; scans give it its offsets.
     int my_cnt[BR_NQUEUES], my_off[BR_NQUEUES], my_comb = 0, my_slots = 0;
 #pragma unroll
     for (int q = 0; q < BR_NQUEUES; ++q) my_cnt[q] = 0;
-    for (int tt = 0; tt * T < Lq; ++tt) {
-        const int ns = walk_pieces(tid, tt, chunk, segs, [&](int, int, int, int q) { bump(my_cnt, q); });
-        my_comb += ns > 1;
-        my_slots += ns > 1 ? ns : 0;
-    }
+    for_my_sequences([&](int b, int Lq) {
+        for (int tt = 0; tt * T < Lq; ++tt) {
+            const int ns = walk_pieces(b, tt, chunk, segs, [&](int, int, int, int q) { bump(my_cnt, q); });
+            my_comb += ns > 1;
+            my_slots += ns > 1 ? ns : 0;
+        }
+    });
     // (all eleven counts through one scan)
     __shared__ int s_scan[(BR_NQUEUES + 2) * (kPlanThreads / 64)];
     int sc[BR_NQUEUES + 2], sc_tot[BR_NQUEUES + 2];
@@ -466,21 +478,19 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             }
         }
     }
-    // The query blocks' pieces (the thread of every sequence; the offsets of the counting pass above).
-    if (tid < B) {
-        const int b = tid;
+    // The query blocks' pieces (the thread of every sequence, in the order and at the offsets of the counting pass above).
+    int pos[BR_NQUEUES];
+#pragma unroll
+    for (int q = 0; q < BR_NQUEUES; ++q) pos[q] = s_base[q] + my_off[q];
+    int slot = off_slot, ci = off_comb;
+    for_my_sequences([&](int b, int L) {
         const int pq = b * M + M - 1;
-        const int L = len[pq];
         BrItem it;
         it.b = b; it.m = M - 1; it.pe = br_prev_blocks(M - 1, M);
         it.len_m = L; it.start_m = start[pq]; it.len0 = len[b * M]; it.start0 = start[b * M];
         it.tok_m = tok[pq]; it.tok0 = tok[b * M];
         it.pad[0] = it.pad[1] = 0;
         it.nprev = M > 1 ? prev_tiles[b] : 0;
-        int pos[BR_NQUEUES];
-#pragma unroll
-        for (int q = 0; q < BR_NQUEUES; ++q) pos[q] = s_base[q] + my_off[q];
-        int slot = off_slot, ci = off_comb;
         for (int tt = 0; tt * T < L; ++tt) {
             const int ns = walk_pieces(b, tt, chunk, segs, no_op);
             if (ns > 1) {
@@ -497,7 +507,7 @@ __global__ __launch_bounds__(kPlanThreads) void br_plan_kernel(int* __restrict__
             });
             if (ns > 1) slot += ns;
         }
-    }
+    });
 }
 
 // Block table straight from per-block lengths (left- or right-aligned spans): the packed-layout

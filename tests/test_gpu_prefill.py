@@ -129,6 +129,17 @@ def test_repeated_calls_reuse_the_plan():
     assert plan[48].item() == 0 and (plan[32:41] == 0).all()     # done and ticket counters re-armed
 
 
+def test_more_sequences_than_plan_threads():
+    # the plan kernel walks one sequence per thread; a batch beyond its 512 threads takes the looping path (the
+    # sequences whose blocks straddle two queues' runs have their query block's walk cut in two: partial slots and
+    # merges come from both rounds of the loop)
+    rng = np.random.default_rng(7)
+    B = 600
+    blocks = [[int(rng.integers(0, 20)), int(rng.integers(0, 40)), int(rng.integers(1, 40)), int(rng.integers(1, 33))] for _ in range(B)]
+    lay = synthetic.make_layout(blocks)
+    check(lay, 4, 2, 64, torch.bfloat16, seed=11)
+
+
 def test_config2_full_size():
     # Mistral-7B-shaped layer: B=4, 32/8 heads, D=128, 64 + 20 x 160 + 32 tokens, projections + RoPE
     lay = synthetic.uniform_layout(4, 64, 20, 160, 32)
