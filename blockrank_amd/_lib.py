@@ -18,6 +18,7 @@ BR_DTYPE_F16 = 2
 BR_ERR_ARG = 1
 BR_ERR_SPACE = 2
 BR_ERR_HIP = 3
+BR_ERR_PLAN = 4
 
 _I64x3 = c_int64 * 3
 
@@ -36,6 +37,8 @@ SIGNATURES = {
     "br_last_error": (c_char_p, []),
     "br_tile_tokens": (c_int, [c_int, c_int]),
     "br_plan_ints": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "br_plan_check": (c_int, [c_void_p, c_void_p]),
+    "br_plan_rearm": (c_int, [c_void_p, c_void_p]),
     "br_plan_build": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "br_plan_build_from_lengths": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "br_plan_build_packed": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -168,6 +168,23 @@ class BlockMask:
             self._plans[key] = plan
         return plan
 
+    def plans_at_rest(self) -> bool:
+        """Whether every plan built for this mask is ready for a launch (waits for the device).  A launch that did not
+        run to its end leaves a plan's ticket counters counting; ``rearm_plans`` puts them back."""
+        lib = _lib.load()
+        for plan in self._plans.values():
+            rc = lib.br_plan_check(plan.data_ptr(), _stream_ptr(self.device))
+            if rc == _lib.BR_ERR_PLAN:
+                return False
+            _lib.check(rc)
+        return True
+
+    def rearm_plans(self) -> None:
+        lib = _lib.load()
+        with torch.cuda.device(self.device):
+            for plan in self._plans.values():
+                _lib.check(lib.br_plan_rearm(plan.data_ptr(), _stream_ptr(self.device)))
+
     def block_lengths(self) -> torch.Tensor:
         """(B, M) int32 number of real tokens per block."""
         return self.lengths if self.lengths is not None else self.valid.sum(-1, dtype=torch.int32)

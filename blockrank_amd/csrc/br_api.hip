@@ -9,6 +9,7 @@
 #include "br_common.h"
 #include "br_score_tiles.h"
 
+void br_launch_plan_rearm(int* plan, hipStream_t stream);
 void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int pool,
                     int* plan, hipStream_t stream);
 int br_launch_prefill_bf16(const BrPrefillParams& p, int D, int NW, int n_cu, int combine_grid, hipStream_t stream,
@@ -168,6 +169,28 @@ size_t br_plan_ints(int B, int M, int H, int Nq, int Nkv) {
     int nw;
     if (!make_geom(Nq, Nkv, &g, &nw) || B <= 0 || M <= 0 || H <= 0) return 0;
     return br_plan_total_ints(B, M, H, br_tokens_per_tile(g));
+}
+
+int br_plan_check(const int32_t* plan, void* stream) {
+    if (!plan) return fail(BR_ERR_ARG, "null pointer");
+    int32_t words[BR_PH_DONE - BR_PH_QTICKET + 1];
+    hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (e == hipSuccess) e = hipMemcpy(words, plan + BR_PH_QTICKET, sizeof(words), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return fail(BR_ERR_HIP, "reading the plan header: %s", hipGetErrorString(e));
+    for (int i = 0; i < BR_NQUEUES; ++i)
+        if (words[i] != 0)
+            return fail(BR_ERR_PLAN, "plan not at rest: ticket counter of queue %d is %d (a launch on it did not run to its end); call br_plan_rearm",
+                        i, (int)words[i]);
+    if (words[BR_PH_DONE - BR_PH_QTICKET] != 0)
+        return fail(BR_ERR_PLAN, "plan not at rest: %d workgroups of a launch have left and the others have not; call br_plan_rearm",
+                    (int)words[BR_PH_DONE - BR_PH_QTICKET]);
+    return BR_OK;
+}
+
+int br_plan_rearm(int32_t* plan, void* stream) {
+    if (!plan) return fail(BR_ERR_ARG, "null pointer");
+    br_launch_plan_rearm(plan, static_cast<hipStream_t>(stream));
+    return check_launch("br_plan_rearm");
 }
 
 // Address of this device's copy of the scratch array, looked up once per device (with that device current).

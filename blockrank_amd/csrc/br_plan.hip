@@ -522,7 +522,19 @@ __global__ void br_block_table_from_len_kernel(const int* __restrict__ lens, int
     start[p] = left_padded ? H - l : 0;
 }
 
+// Ticket counters and the count of workgroups that have left back to zero (what the last workgroup of a launch that
+// ran to its end does itself).
+__global__ void br_plan_rearm_kernel(int* __restrict__ plan) {
+    const int i = threadIdx.x;
+    if (i < BR_NQUEUES) plan[BR_PH_QTICKET + i] = 0;
+    if (i == BR_NQUEUES) plan[BR_PH_DONE] = 0;
+}
+
 }  // namespace
+
+void br_launch_plan_rearm(int* plan, hipStream_t stream) {
+    hipLaunchKernelGGL(br_plan_rearm_kernel, dim3(1), dim3(64), 0, stream, plan);
+}
 
 void br_launch_plan(const uint8_t* valid, const int* lens, int left_padded, int packed, int B, int M, int H, int T, int par, int pool,
                     int* plan, hipStream_t stream) {

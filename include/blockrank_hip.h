@@ -31,6 +31,7 @@ extern "C" {
 #define BR_ERR_ARG 1      /* bad shape, dtype, alignment or null pointer (reference: AssertionError) */
 #define BR_ERR_SPACE 2    /* a caller-provided buffer is too small */
 #define BR_ERR_HIP 3      /* a HIP runtime call or launch failed */
+#define BR_ERR_PLAN 4     /* br_plan_check: the plan's launch counters are not at rest */
 
 /* Library version, major*10000 + minor*100 + patch. */
 int br_version(void);
@@ -44,6 +45,15 @@ int br_tile_tokens(int Nq, int Nkv);
 
 /* Size, in int32 elements, of the plan buffer for a (B, M, H) batch with this head layout. */
 size_t br_plan_ints(int B, int M, int H, int Nq, int Nkv);
+
+/* A plan carries the ticket counters of the persistent attention kernel; the last workgroup of every launch puts them
+ * back to zero.  A launch that did not run to its end (a fault, a killed process sharing the buffer) leaves them
+ * counting, and the next launch on that plan would hand out no work.  br_plan_check waits for `stream`, reads the
+ * counters back and returns BR_OK or BR_ERR_PLAN (the only entry point that synchronises: for diagnostics, not for
+ * the serving path); br_plan_rearm enqueues their reset (a small kernel: safe under graph capture).  No reference
+ * counterpart: its mask tensor has no state. */
+int br_plan_check(const int32_t* plan, void* stream);
+int br_plan_rearm(int32_t* plan, void* stream);
 
 /* Build the request plan (block table + work items) from the (B, M, H) block mask, one byte per
  * token slot, non-zero = real token.  Replaces eager_blockrank_attention_mask /

@@ -129,6 +129,21 @@ def test_repeated_calls_reuse_the_plan():
     assert plan[48].item() == 0 and (plan[32:41] == 0).all()     # done and ticket counters re-armed
 
 
+def test_plan_left_by_an_unfinished_launch_is_detected_and_rearmed():
+    lay = synthetic.make_layout([[64] + [100] * 6 + [40]] * 2)
+    q, k, v = synthetic.random_qkv(lay, 8, 2, 128, torch.bfloat16, DEV, seed=8)
+    bm = br.BlockMask(lay.valid.to(DEV))
+    want = br.blockrank_attention(q, k, v, bm, 0.09)
+    assert bm.plans_at_rest()
+    plan = bm.plan(8, 2)
+    plan[33] = 7                      # what a launch that never finished leaves behind: tickets handed out, nobody home
+    plan[48] = 3
+    assert not bm.plans_at_rest()
+    bm.rearm_plans()
+    assert bm.plans_at_rest()
+    assert torch.equal(br.blockrank_attention(q, k, v, bm, 0.09), want)
+
+
 def test_more_sequences_than_plan_threads():
     # the plan kernel walks one sequence per thread; a batch beyond its 512 threads takes the looping path (the
     # sequences whose blocks straddle two queues' runs have their query block's walk cut in two: partial slots and
