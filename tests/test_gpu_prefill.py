@@ -144,12 +144,13 @@ def test_plan_left_by_an_unfinished_launch_is_detected_and_rearmed():
     assert torch.equal(br.blockrank_attention(q, k, v, bm, 0.09), want)
 
 
-def test_more_sequences_than_plan_threads():
+@pytest.mark.parametrize("B", [600, 2100])
+def test_more_sequences_than_plan_threads(B):
     # the plan kernel walks one sequence per thread; a batch beyond its 512 threads takes the looping path (the
     # sequences whose blocks straddle two queues' runs have their query block's walk cut in two: partial slots and
     # merges come from both rounds of the loop)
+    # (2100 sequences of four blocks are also more blocks than the plan kernel stages in LDS)
     rng = np.random.default_rng(7)
-    B = 600
     blocks = [[int(rng.integers(0, 20)), int(rng.integers(0, 40)), int(rng.integers(1, 40)), int(rng.integers(1, 33))] for _ in range(B)]
     lay = synthetic.make_layout(blocks)
     check(lay, 4, 2, 64, torch.bfloat16, seed=11)
